@@ -1,0 +1,63 @@
+"""Argument marshalling for one megakernel launch.
+
+The positional order is the boundary contract of reference
+``megakernels/demos/latency/mk.py:15-49`` (and of the binding it calls,
+``demos/low-latency-llama/llama.cu:28-52``): barriers, instructions, timings,
+nine weight tensors, K and V caches viewed as ``[(L B), T, KVH, D]``, the two
+rope tables, seven activation buffers, then ``pos_id``, ``attn_scale``,
+``rms_norm_eps``, ``skip_attn_reduction`` and the keyword ``stream``.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from megakernels_amd.demos.latency.instructions import Globals
+from megakernels_amd.mk import MK_Interpreter
+
+
+def interpret_with_mk(globs: Globals, mk_func):
+    # [L, B, T, KVH, D] -> [(L B), T, KVH, D]; a view, the cache is contiguous
+    k_cache_4d = globs.k_cache.flatten(0, 1)
+    v_cache_4d = globs.v_cache.flatten(0, 1)
+
+    mk_func(
+        # vm state
+        globs.barriers,
+        globs.instructions,
+        globs.timings,
+        # weights
+        globs.qkv_proj_weights,
+        globs.attn_ln_weights,
+        globs.o_proj_weights,
+        globs.mlp_ln_weights,
+        globs.up_proj_weights,
+        globs.gate_proj_weights,
+        globs.down_proj_weights,
+        globs.lm_head_norm_weights.data,
+        globs.lm_head_weights.data,
+        k_cache_4d,
+        v_cache_4d,
+        # rope
+        globs.rope_cos,
+        globs.rope_sin,
+        # activations
+        globs.hidden_states,
+        globs.post_ln_rope_q,
+        globs.attn_out,
+        globs.attn_lse_intermediates,
+        globs.attn_out_intermediates,
+        globs.silu_out,
+        globs.logits,
+        # scalars
+        globs.pos_id,
+        globs.attn_scale,
+        globs.rms_norm_eps,
+        globs.skip_attn_reduction,
+        stream=torch.cuda.current_stream(),
+    )
+
+
+class LatencyMK_Interpreter(MK_Interpreter):
+    def interpret(self, globs: Globals):
+        interpret_with_mk(globs, self.mk_func)

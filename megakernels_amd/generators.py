@@ -1,0 +1,108 @@
+"""Token generation loops (reference ``megakernels/generators.py``).
+
+``MK_Generator.run`` is the per-token hot loop of the ``mk`` path
+(``generators.py:121-143``): embedding row into ``hidden_states``, barrier
+reset, ``pos_id`` update, one megakernel launch, ``argmax`` over the bf16
+logits (first maximum wins).  Nothing in it synchronises with the host.
+"""
+
+from __future__ import annotations
+
+import torch
+from torch import Tensor
+
+from megakernels_amd.mk import MK_Interpreter
+from megakernels_amd.model_types import BatchState
+from megakernels_amd.scheduler import Schedule
+
+
+class Generator:
+    def generate(self, output_tokens: Tensor, prompt_len: int, ntok: int, ntok_already_generated: int = 1):
+        raise NotImplementedError
+
+    def generate_with_eos(
+        self,
+        output_tokens: Tensor,
+        prompt_len: int,
+        ntok: int,
+        eos_token_check_interval: int,
+        eos_token_ids: list[int],
+    ):
+        """Decode in chunks of ``eos_token_check_interval`` tokens and look for
+        an end-of-sequence id on the host after each chunk.  Returns
+        ``(index of the first eos token or ntok, tokens generated)``
+        (reference ``generators.py:21-58``)."""
+        assert output_tokens.shape[0] == 1, "batch size must be 1"
+        for done in range(1, ntok, eos_token_check_interval):
+            chunk = min(eos_token_check_interval, ntok - done)
+            self.generate(output_tokens, prompt_len=prompt_len, ntok=chunk, ntok_already_generated=done)
+            for j, token in enumerate(output_tokens[0, done : done + chunk].cpu().tolist()):
+                if token in eos_token_ids:
+                    # the first token came from prefill, hence the -1
+                    return done + j, done + chunk - 1
+        return ntok, ntok - 1
+
+
+class PyTorchGenerator(Generator):
+    """Plain PyTorch decode, one dense forward per token
+    (reference ``generators.py:61-92``)."""
+
+    def __init__(self, model):
+        self.model = model
+
+    def generate(self, output_tokens: Tensor, prompt_len: int, ntok: int, ntok_already_generated: int = 1):
+        first_seq_len = prompt_len + ntok_already_generated
+        for i in range(ntok):
+            src = i + ntok_already_generated - 1
+            state = BatchState(
+                input_ids=output_tokens[:, src : src + 1],
+                position_ids=torch.tensor([first_seq_len - 1 + i], device=self.model.device),
+                seq_len=first_seq_len + i,
+            )
+            out = self.model(state)
+            output_tokens[:, src + 1] = out.output_ids.squeeze(-1)
+
+
+class MK_Generator(Generator):
+    def __init__(
+        self,
+        model,
+        interpreter: MK_Interpreter,
+        schedule: Schedule,
+        barrier_fill_val: int = 0,
+        skip_mk: bool = False,
+        skip_rest: bool = False,
+    ):
+        self.model = model
+        self.interpreter = interpreter
+        self.schedule = schedule
+        self.barrier_fill_val = barrier_fill_val
+        self.skip_mk = skip_mk
+        self.skip_rest = skip_rest
+        self.fill()
+
+    def fill(self):
+        self.schedule.globs.barriers.fill_(self.barrier_fill_val)
+
+    def replace_with_noops(self):
+        self.schedule.globs.instructions.zero_()
+
+    def run(self, input_ids: Tensor, pos_id: int):
+        globs = self.schedule.globs
+        if not self.skip_rest:
+            embedded = self.model.model.embed_tokens(BatchState(input_ids=input_ids))
+            globs.hidden_states[:] = embedded.hidden_states.reshape(-1)
+        self.fill()
+        globs.pos_id = pos_id
+        if not self.skip_mk:
+            self.interpreter.interpret(globs)
+        if self.skip_rest:
+            return input_ids
+        return torch.argmax(globs.logits, dim=-1)
+
+    def generate(self, output_tokens: Tensor, prompt_len: int, ntok: int, ntok_already_generated: int = 1):
+        for i in range(ntok):
+            src = ntok_already_generated + i - 1
+            pos_id = prompt_len + ntok_already_generated + i - 1
+            output_ids = self.run(output_tokens[:, src : src + 1], pos_id=pos_id)
+            output_tokens[:, src + 1] = output_ids.reshape(-1)
