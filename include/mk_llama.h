@@ -1,0 +1,117 @@
+/*
+ * C ABI of the MI355X batch-1 decode megakernel (libmk_llama.so).
+ *
+ * This is the drop-in boundary of the reference's `mk` path: what the
+ * reference's Python calls through the pybind module `mk_llama`
+ * (megakernels/demos/latency/mk.py:15-49 -> demos/low-latency-llama/llama.cu:26-52
+ * -> __global__ mk<...>, include/megakernel.cuh:166-171).  One call launches one
+ * persistent HIP kernel - one workgroup per compute unit, workgroup w running
+ * instructions[w, 0..num_slots) in order - asynchronously on the given stream.
+ *
+ * Plain pointers and sizes only; the caller (PyTorch in the shipped host code)
+ * owns every buffer.  All tensors are contiguous device memory.  bf16 tensors
+ * are passed as uint16_t bit patterns.
+ */
+#ifndef MK_LLAMA_H
+#define MK_LLAMA_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MK_LLAMA_ABI_VERSION 1
+#define MK_INSTRUCTION_WORDS 32   /* megakernels/scheduler.py:13, include/config.cuh:14 */
+#define MK_TIMING_SLOTS 128       /* megakernels/scheduler.py:14, include/config.cuh:18 */
+#define MK_BARRIER_ROWS 10        /* megakernels/demos/latency/scheduler.py:53-61 */
+
+/* Status codes written by the kernel into the workspace and returned by
+ * mk_llama_read_status(). */
+enum {
+    MK_STATUS_OK = 0,
+    MK_STATUS_BARRIER_TIMEOUT = 1,   /* a barrier wait exceeded spin_limit_us */
+    MK_STATUS_BAD_OPCODE = 2,        /* reference: asm trap, include/util.cuh:38 */
+    MK_STATUS_ATTN_TOO_LONG = 3,     /* one attention partition exceeds the on-chip score buffer */
+    MK_STATUS_BAD_INSTRUCTION = 4    /* field out of range for the given shapes */
+};
+
+/* Arguments of one launch, in the positional order of the reference binding
+ * (megakernels/demos/latency/mk.py:17-48), followed by the shapes the
+ * reference bakes in at compile time (demos/low-latency-llama/llama.cuh:15-24,149-158). */
+typedef struct mk_llama_args {
+    /* VM state */
+    int32_t *barriers;              /* [L, 10, H + 2 KVH]; read-modify-write */
+    const int32_t *instructions;    /* [num_workers, num_slots, 32] */
+    int32_t *timings;               /* [num_workers, num_slots, 128]; may be NULL */
+    /* weights */
+    const uint16_t *qkv_weights;          /* [L, (H + 2 KVH) D, hidden] */
+    const uint16_t *attn_norm_weights;    /* [L, hidden] */
+    const uint16_t *o_weights;            /* [L, hidden, H D] */
+    const uint16_t *mlp_norm_weights;     /* [L, hidden] */
+    const uint16_t *up_weights;           /* [L, inter, hidden] */
+    const uint16_t *gate_weights;         /* [L, inter, hidden] */
+    const uint16_t *down_weights;         /* [L, hidden, inter] */
+    const uint16_t *lm_head_norm_weights; /* [hidden] */
+    const uint16_t *lm_head_weights;      /* [vocab, hidden] */
+    uint16_t *k_cache;                    /* [L, kv_max_len, KVH, D]; row pos_id is written */
+    uint16_t *v_cache;
+    const float *rope_cos;                /* [rope_positions, D], rotary pairs adjacent */
+    const float *rope_sin;
+    /* activations */
+    uint16_t *hidden_states;              /* [hidden]; in: embedding row, out: final hidden state */
+    uint16_t *q_post_rope;                /* [H D] */
+    uint16_t *attn_out;                   /* [H D] */
+    float *attn_lse_intermediates;        /* [H, max_partials] */
+    float *attn_out_intermediates;        /* [H, max_partials, D] */
+    uint16_t *silu_out;                   /* [inter] */
+    uint16_t *logits;                     /* [vocab] */
+    /* scalars of the reference call */
+    int32_t pos_id;
+    float attn_scale;
+    float rms_norm_eps;
+    int32_t skip_attn_reduction;
+    /* shapes */
+    int32_t num_layers, hidden_size, intermediate_size;
+    int32_t num_attention_heads, num_kv_heads, head_dim, vocab_size;
+    int32_t num_workers, num_slots;       /* instruction tensor dims 0 and 1 */
+    int32_t kv_max_len, max_partials, rope_positions;
+    int32_t matvec_reduction_size;        /* column-group width, 2048 in the reference */
+    int32_t attn_reduction_size;          /* heads per reduction instruction, 4 */
+    /* runtime */
+    void *workspace;                      /* mk_llama_workspace_bytes() bytes, zeroed once by the caller */
+    uint64_t workspace_bytes;
+    uint32_t spin_limit_us;               /* give up a barrier wait after this long; 0 = default (2 s) */
+    uint32_t flags;                       /* reserved, 0 */
+} mk_llama_args;
+
+/* Bytes of scratch device memory a launch needs for these shapes.  The caller
+ * zeroes it once; the kernel leaves it clean after every successful launch.
+ * Holds sharded barrier counters, residual partial sums and the status block. */
+uint64_t mk_llama_workspace_bytes(int32_t num_layers, int32_t hidden_size, int32_t intermediate_size,
+                                  int32_t matvec_reduction_size);
+
+/* Validates the arguments against what the kernel assumes, then launches on
+ * `hip_stream` (a hipStream_t, NULL = default stream) without synchronising.
+ * Returns 0 or a negative error; the message is available from
+ * mk_llama_last_error().  Replaces the `mk_llama(...)` call of
+ * megakernels/demos/latency/mk.py:15-49. */
+int mk_llama_launch(const mk_llama_args *args, void *hip_stream);
+
+/* Synchronises `hip_stream` and copies the 4-word status block
+ * {code, worker, slot, opcode} of the workspace to the host.  A non-zero code
+ * means the launch gave up; the workspace must then be zeroed again. */
+int mk_llama_read_status(void *workspace, void *hip_stream, int32_t out[4]);
+
+/* what = 0: compute units of the current device; 1: LDS bytes the kernel
+ * requests per workgroup; 2: threads per workgroup; 3: ABI version; 4: longest
+ * attention partition (tokens) the kernel accepts. */
+int mk_llama_query(int what);
+
+const char *mk_llama_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

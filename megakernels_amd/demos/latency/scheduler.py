@@ -124,7 +124,7 @@ def make_globals(model, skip_attn_reduction: bool = True) -> Globals:
         down_proj_block_size=16,
         o_proj_block_size=16,
         lm_head_block_size=16,
-        matvec_reduction_size=2048,
+        matvec_reduction_size=min(2048, config.hidden_size),
         qkv_block_size=16,
         attn_kv_block_size=16,
         attn_reduction_size=4,

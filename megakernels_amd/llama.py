@@ -405,6 +405,28 @@ class LlamaForCausalLM:
         model.setup_caches()
         return model
 
+    def to(self, device: DeviceType) -> "LlamaForCausalLM":
+        """A copy of the model (weights, rope tables, fresh zeroed KV cache) on
+        ``device``; a tied LM head stays tied."""
+        emb = self.model.embed_tokens.weight
+        head = self.lm_head.lm_head.weight
+        return type(self)._assemble_moved(self, torch.device(device), head is emb)
+
+    @classmethod
+    def _assemble_moved(cls, src: "LlamaForCausalLM", device, tied: bool):
+        def move(t):
+            return t.to(device).contiguous()
+
+        stacked = StackedParams(**{k: move(v) for k, v in vars(src.stacked_params).items()})
+        embed = move(src.model.embed_tokens.weight)
+        head = embed if tied else move(src.lm_head.lm_head.weight)
+        model = cls(
+            src.config, src.extra_config, stacked, embed, move(src.lm_head.input_norm.weight), head,
+            move(src.model.rope_cos), move(src.model.rope_sin),
+        )
+        model.setup_caches()
+        return model
+
     def setup_caches(self):
         """Zeroed K and V caches ``[L, batch, max_len, KVH, D]``
         (reference ``llama.py:552-567``)."""
