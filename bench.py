@@ -1,0 +1,233 @@
+"""Headline benchmark: batch-1 greedy decode through the HIP megakernel.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2]
+
+One "step" is one decode step (one token): embedding row -> hidden state,
+barrier reset, ONE megakernel launch, argmax over the logits, token write -
+the per-token loop of the reference's mk generator
+(megakernels/generators.py:121-163).  Weights, KV cache and instruction
+tensor are resident in HBM before the timed region starts.
+
+Workloads (all Llama-3.2-1B architecture, random bf16 weights N(0, 0.02) from
+seed 0, RMSNorm weights 1):
+  c1  32-token prompt prefilled by the plain PyTorch forward, decode from position 32
+  c2  KV cache pre-filled to 4096 positions with seeded N(0,1), decode from position 4096  (default)
+  c3  KV cache pre-filled to 16384 positions
+
+Prints one JSON line.  `roofline` prices the megakernel alone: algorithmic
+bytes per launch (weights + norm weights + K/V read) divided by the mean
+kernel time measured with events on the launch stream.  `cpu_baseline` is the
+C restatement of the reference's Python VM (the parity checker) timed on this
+host's cores over a bounded number of the same decode steps; its tokens are
+also compared with the GPU's.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def algorithmic_bytes(cfg, pos: int) -> int:
+    """Bytes one decode step must read at least: bf16 matrices (tied embedding
+    counted once as the LM head), norm weights, and K/V of positions 0..pos.
+    Left out: embedding row, KV append, logits write, rope row, activations,
+    instructions, barriers."""
+    L, hid, inter = cfg.num_hidden_layers, cfg.hidden_size, cfg.intermediate_size
+    H, KVH, D = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    matrices = L * ((H + 2 * KVH) * D * hid + hid * hid + 3 * inter * hid) + cfg.vocab_size * hid
+    norms = (2 * L + 1) * hid
+    kv = L * 2 * KVH * D * (pos + 1)
+    return 2 * (matrices + norms + kv)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3"])
+    ap.add_argument("--cpu-steps", type=int, default=32, help="decode steps timed on the CPU checker (0 = skip)")
+    ap.add_argument("--sched", default="rr")
+    ap.add_argument("--partitions", type=int, default=0, help="attention partitions (0 = one per 256 positions, max 24)")
+    args = ap.parse_args()
+
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs the decode path on ONE GPU; --gpus N with N > 1 is not supported "
+              "(batch-1 decode does not shard into independent units)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from megakernels_amd.demos.latency.scheduler import LatencyScheduleBuilder, pick_num_attention_partitions
+    from megakernels_amd.dispatch import make_mk_interpreter
+    from megakernels_amd.generators import MK_Generator
+    from megakernels_amd.llama import LlamaConfig, LlamaForCausalLM
+    from megakernels_amd.model_types import BatchState, ExtraModelConfig
+    from megakernels_amd.scheduler import assign_to_sms, tensorize_instructions
+    from megakernels_amd.utils import get_sm_count, set_sm_count_override
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    cfg = LlamaConfig.llama_1b()
+    total_steps = args.warmup + args.steps
+    prefill = {"c1": 32, "c2": 4096, "c3": 16384}[args.workload]
+    max_len = prefill + total_steps + 16
+    t_setup = time.time()
+    model_cpu = LlamaForCausalLM.from_random(cfg, ExtraModelConfig(interleave_rope=True, max_len_override=max_len), seed=0)
+
+    prompt_gen = torch.Generator().manual_seed(1)
+    prompt = torch.randint(0, cfg.vocab_size, (1, 32), generator=prompt_gen)
+    if args.workload == "c1":
+        # prefill once with the plain forward; both the GPU and the checker start from its cache
+        out = model_cpu(BatchState(input_ids=prompt, position_ids=torch.arange(32)))
+        first_token = int(out.output_ids[0, -1])
+    else:
+        kv_gen = torch.Generator().manual_seed(2)
+        for cache in model_cpu.stacked_kv_cache:
+            shape = list(cache.shape)
+            shape[2] = prefill
+            cache[:, :, :prefill] = torch.randn(shape, generator=kv_gen).to(cache.dtype)
+        first_token = int(prompt[0, 0])
+
+    workers = get_sm_count(device)
+    set_sm_count_override(workers)
+    partitions = args.partitions or pick_num_attention_partitions(prefill, total_steps)
+    model = model_cpu.to(device)
+    for dst, src in zip(model.stacked_kv_cache, model_cpu.stacked_kv_cache):
+        dst.copy_(src)
+
+    schedule = LatencyScheduleBuilder.build(model, num_attention_partitions=partitions)
+    tensorize_instructions(schedule.globs, assign_to_sms(args.sched, schedule=schedule))
+    interpreter = make_mk_interpreter("latency")
+    gen = MK_Generator(model, interpreter, schedule)
+    mk_mod = sys.modules["mk_llama"]
+
+    ntok = total_steps + 1
+    output_tokens = torch.zeros(1, ntok, device=device, dtype=torch.long)
+    output_tokens[0, 0] = first_token
+    torch.cuda.synchronize()
+    setup_s = time.time() - t_setup
+
+    # ---- warmup -------------------------------------------------------------
+    if args.warmup:
+        gen.generate(output_tokens, prompt_len=prefill, ntok=args.warmup, ntok_already_generated=1)
+    torch.cuda.synchronize()
+    mk_mod.check_status(device)
+
+    # ---- timed region: exactly K steps --------------------------------------
+    # kernel-only events: wrap the interpreter so each launch is bracketed on the launch stream
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    counter = {"i": 0}
+    plain_interpret = interpreter.interpret
+
+    def timed_interpret(globs):
+        i = counter["i"]
+        starts[i].record()
+        plain_interpret(globs)
+        ends[i].record()
+        counter["i"] = i + 1
+
+    interpreter.interpret = timed_interpret
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    gen.generate(output_tokens, prompt_len=prefill, ntok=args.steps, ntok_already_generated=1 + args.warmup)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    interpreter.interpret = plain_interpret
+    mk_mod.check_status(device)
+
+    kernel_ms = [s.elapsed_time(e) for s, e in zip(starts, ends)]
+    kernel_ms_mean = sum(kernel_ms) / len(kernel_ms)
+    first_pos = prefill + args.warmup
+    bytes_per_step = sum(algorithmic_bytes(cfg, first_pos + i) for i in range(args.steps)) / args.steps
+    achieved_gbps = bytes_per_step / (kernel_ms_mean * 1e-3) / 1e9
+
+    tokens_gpu = output_tokens[0].cpu().tolist()
+
+    # ---- CPU baseline: the checker on the same decode steps (bounded sample) --
+    cpu_baseline = None
+    parity = None
+    if args.cpu_steps > 0:
+        from oracle import pyvm
+
+        n_cpu = min(args.cpu_steps, total_steps)
+        set_sm_count_override(workers)
+        schedule_cpu = LatencyScheduleBuilder.build(model_cpu, num_attention_partitions=partitions)
+        oracle_gen = pyvm.OracleGenerator(model_cpu, schedule_cpu)
+        tokens_cpu = torch.zeros(1, n_cpu + 1, dtype=torch.long)
+        tokens_cpu[0, 0] = first_token
+        tc0 = time.perf_counter()
+        oracle_gen.generate(tokens_cpu, prompt_len=prefill, ntok=n_cpu, ntok_already_generated=1)
+        cpu_elapsed = time.perf_counter() - tc0
+        cpu_baseline = {
+            "value": round(n_cpu / cpu_elapsed, 3),
+            "unit": "tokens/s",
+            "cores": pyvm.threads(),
+            "kind": "port",
+            "sample": f"first {n_cpu} decode steps of the same workload on the C restatement of the Python VM "
+                      f"(OpenMP, {pyvm.threads()} threads), {cpu_elapsed:.1f} s",
+            "us_per_step": round(cpu_elapsed / n_cpu * 1e6, 1),
+        }
+        expect = tokens_cpu[0].tolist()
+        got = tokens_gpu[: n_cpu + 1]
+        agree = sum(int(a == b) for a, b in zip(expect, got))
+        parity = {"tokens_compared": n_cpu + 1, "tokens_equal": agree, "bit_exact": agree == n_cpu + 1}
+
+    result = {
+        "metric": "batch-1 decode tokens/s (Llama-3.2-1B arch)",
+        "value": round(args.steps / elapsed, 2),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(elapsed / args.steps * 1e3, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.workload}: Llama-3.2-1B architecture, random-init bf16 weights (seed 0), batch 1, "
+                        f"KV pre-filled to {prefill} positions, greedy decode of {args.steps} timed tokens "
+                        f"from position {first_pos}",
+            "workers": workers,
+            "attention_partitions": partitions,
+            "assignment": args.sched,
+            "instructions_per_step": len(schedule.dag_nodes),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(achieved_gbps, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved_gbps / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "kernel": "mk_llama_kernel<4,4,64>",
+            "kernel_us": round(kernel_ms_mean * 1e3, 2),
+            "algorithmic_bytes_per_launch": int(bytes_per_step),
+        },
+        "cpu_baseline": cpu_baseline,
+        "parity": parity,
+        "whole_step_roofline_frac": round(bytes_per_step / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS, 4),
+        "setup_s": round(setup_s, 1),
+    }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
