@@ -27,6 +27,11 @@ extern "C" {
 #define MK_TIMING_SLOTS 128       /* megakernels/scheduler.py:14, include/config.cuh:18 */
 #define MK_BARRIER_ROWS 10        /* megakernels/demos/latency/scheduler.py:53-61 */
 
+/* args.flags: record per-instruction timings into `timings` (slot 0 start, 1 dependency ready,
+ * 2 matvec done, 3 end - ticks of the 100 MHz wall clock since the workgroup started; slot 4 opcode).
+ * Counterpart of the reference's compile-time TIMING_RECORD_ENABLED (include/config.cuh:46). */
+#define MK_FLAG_TIMINGS 1u
+
 /* Status codes written by the kernel into the workspace and returned by
  * mk_llama_read_status(). */
 enum {
@@ -83,7 +88,7 @@ typedef struct mk_llama_args {
     void *workspace;                      /* mk_llama_workspace_bytes() bytes, zeroed once by the caller */
     uint64_t workspace_bytes;
     uint32_t spin_limit_us;               /* give up a barrier wait after this long; 0 = default (2 s) */
-    uint32_t flags;                       /* reserved, 0 */
+    uint32_t flags;                       /* MK_FLAG_* */
 } mk_llama_args;
 
 /* Bytes of scratch device memory a launch needs for these shapes.  The caller

@@ -2,19 +2,25 @@
 //
 // Execution model (counterpart of the reference VM runtime, include/megakernel.cuh:15-171,
 // include/controller/controller.cuh:24-132, include/util.cuh:260-304, rebuilt for CDNA4):
-//   * grid = one workgroup per compute unit, 1024 threads = 16 wave64; workgroup w executes
-//     instructions[w, 0..num_slots) strictly in order.  An LDS request above half the CU's
-//     160 KB keeps a second workgroup off the same CU.
-//   * there are no specialised loader / storer / controller wavefronts: every wave issues its
-//     own 16-byte global loads and keeps several weight rows in flight in VGPRs.  The first
-//     rows of an instruction are requested BEFORE the instruction waits for its dependency,
-//     because weights never depend on the barrier.
+//   * grid = one workgroup per compute unit; workgroup w executes instructions[w, 0..num_slots)
+//     strictly in order.  The LDS request (> half of the CU's 160 KB) keeps a second workgroup
+//     off the same CU.
+//   * a workgroup is 9 wave64: eight CONSUMER waves stream weight rows (16-byte global loads
+//     straight into VGPRs, several rows in flight per wave, no LDS staging for weights) and do
+//     the dot products; one CONTROLLER wave does everything that is latency-critical and small:
+//     it waits on the dependency counters, fetches the activation vector, normalises it and hands
+//     it to the consumers through LDS, and after the matvec it runs the epilogue (RoPE, SiLU,
+//     residual, stores) and signals the next counter.  The controller never has bulk loads
+//     outstanding, so its polls and 4 KB activation loads do not queue behind its own weight
+//     traffic (vector memory returns in order per wave).  Consumers request the first rows of the
+//     NEXT instruction as soon as they finish the current one, before any dependency is checked:
+//     weights never depend on a barrier.
 //   * cross-CU ordering is only through counters in HBM, with the counts of the reference's
 //     Python VM (megakernels/demos/latency/python_vm.py).  The eight XCDs have private L2
 //     caches, so everything one CU writes for another (activations, the new KV row, counters)
 //     is stored write-through and loaded with agent-scope ("sc1") accesses; no cache-wide
-//     write-back / invalidate is ever issued.  A producer's stores are complete
-//     (s_waitcnt vmcnt(0), part of __syncthreads) before it bumps the counter.
+//     write-back / invalidate is ever issued.  A producer waits for its stores (s_waitcnt
+//     vmcnt(0)) before it bumps the counter.
 //   * the four counters that receive one arrival per worker (barriers[l, 2..5, 0]) are kept
 //     as 16 shards in the workspace while the kernel runs (256 atomics on one address cost
 //     ~3 us, 16 per shard ~0.2 us); the last workgroup to finish adds the shard totals into
@@ -38,20 +44,25 @@
 
 namespace {
 
-constexpr int kThreads = 1024;
-constexpr int kWaves = 16;
+constexpr int kConsumerWaves = 8;
+constexpr int kConsumerThreads = kConsumerWaves * 64;
+constexpr int kThreads = kConsumerThreads + 64;  // + one controller wave
+constexpr int kVirtualWaves = 16;   // attention slot layout is defined for 16 waves; each consumer wave plays two
 constexpr int kShards = 16;         // shards per hot barrier counter
 constexpr int kHotRows = 4;         // barrier rows 2..5 are sharded
 constexpr int kOutRows = 2048;      // rows staged in LDS between matvec and epilogue
+constexpr int kMaxK = 4096;         // longest activation vector handed through LDS
 constexpr int kScoreCap = 6144;     // tokens per attention partition (LDS score buffer)
 constexpr int kMaxHeadDim = 128;
-constexpr int kGqaMax = 4;          // query heads per KV head handled by one attention instruction
+constexpr int kGqa = 4;             // query heads per KV head handled by one attention instruction
 constexpr int kStatusInts = 16;
 constexpr int kDoneSlot = 8;        // workspace int: workgroups finished
 
-// weight rows in flight per wave: bounded by the 128 VGPRs a 1024-thread workgroup leaves each lane
+// Weight rows in flight per consumer wave.  16 VGPRs per 2048-element row; the 9-wave workgroup
+// leaves each lane 168 VGPRs.  8 waves x 4 rows x 4 KB = 128 KB per CU covers the ~4 us a worker
+// spends between two instructions at its ~31 GB/s share of HBM bandwidth.
 template <int KC>
-constexpr int rows_in_flight(int want) { return KC <= 4 ? want : 1; }
+constexpr int rows_in_flight() { return KC <= 4 ? 4 : 2; }
 
 #define AG __HIP_MEMORY_SCOPE_AGENT
 
@@ -85,14 +96,17 @@ struct Smem {
     int last_flag;
     int pad[2];
     int flags[kOutRows / 16];       // per-block "I was the last arriver" (matvec-add)
+    float x[kMaxK];                 // activation vector, lane layout [chunk][lane][8]
     float out[kOutRows];            // matvec row results awaiting the epilogue
-    float wave_max[kWaves][kGqaMax];
-    float wave_l[kWaves][kGqaMax];
-    float head_m[kGqaMax];
-    float head_w[kGqaMax][32];      // reduction weights
-    float wave_o[kWaves][kGqaMax][kMaxHeadDim];
-    float scores[kGqaMax][kScoreCap];
+    float wave_max[kVirtualWaves][kGqa];
+    float wave_l[kVirtualWaves][kGqa];
+    float head_m[kGqa];
+    float head_w[kGqa][32];         // reduction weights
+    float wave_o[kVirtualWaves][kGqa][kMaxHeadDim];
+    float scores[kGqa][kScoreCap];
 };
+static_assert(sizeof(Smem) <= 160 * 1024, "LDS budget");
+static_assert(sizeof(Smem) > 80 * 1024, "must keep a second workgroup off the CU");
 
 // ---------------------------------------------------------------------------------------------
 // agent-coherent memory access (bypass the non-coherent per-XCD L2 contents)
@@ -118,24 +132,130 @@ __device__ __forceinline__ uint4 ld_b128(const void *p) {
 // immutable data (weights, rope tables, old KV rows): ordinary cached 16-byte load
 __device__ __forceinline__ uint4 ld_const_b128(const void *p) { return *(const uint4 *)p; }
 
+// All of this wave's global stores and atomics have been performed.  The "memory" clobber keeps
+// the compiler from moving memory operations across it.
+__device__ __forceinline__ void wait_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void compiler_fence() { asm volatile("" ::: "memory"); }
+
+// Workgroup barrier that orders LDS traffic only: outstanding global loads (the consumers'
+// prefetched weight rows) stay in flight across it.
+__device__ __forceinline__ void wg_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // ---------------------------------------------------------------------------------------------
-// wave-level reductions: xor butterfly in ascending offset order = pairwise tree in lane order
+// wave-level reductions.  The canonical order is a pairwise tree in lane order (an xor butterfly
+// with ascending offsets).  Additions commute exactly, so any exchange pattern that pairs the same
+// partial sums at each level gives the same bits.
 // ---------------------------------------------------------------------------------------------
+// Exchange with lane (l ^ OFFSET) through the VALU data path (DPP within a row of 16 lanes,
+// v_permlane{16,32}_swap across rows) instead of the LDS crossbar, whose ~100-cycle round trip per
+// exchange dominated the reduction-heavy instructions.  Returns the pair {own, partner} in
+// unspecified order, which is all a commutative combine needs.
+struct LanePair {
+    uint32_t a, b;
+};
+template <int OFFSET>
+__device__ __forceinline__ LanePair lane_xor_pair(uint32_t v) {
+    const int vi = (int)v;
+    if constexpr (OFFSET == 1) return {v, (uint32_t)__builtin_amdgcn_update_dpp(0, vi, 0xB1, 0xf, 0xf, false)};
+    else if constexpr (OFFSET == 2) return {v, (uint32_t)__builtin_amdgcn_update_dpp(0, vi, 0x4E, 0xf, 0xf, false)};
+    else if constexpr (OFFSET == 4) {
+        // lanes with bit 2 clear read lane + 4 (row_shl:4, banks 0 and 2), the others lane - 4
+        const int r = __builtin_amdgcn_update_dpp(0, vi, 0x104, 0xf, 0x5, false);
+        return {v, (uint32_t)__builtin_amdgcn_update_dpp(r, vi, 0x114, 0xf, 0xa, false)};
+    } else if constexpr (OFFSET == 8) {
+        return {v, (uint32_t)__builtin_amdgcn_update_dpp(0, vi, 0x128, 0xf, 0xf, false)};  // row_ror:8
+    } else {
+        // a = b = v; the swap exchanges the odd rows (upper half) of a with the even rows (lower
+        // half) of b, leaving own and partner values in a and b.  Written in assembly: the
+        // compiler's builtin for these instructions returns the first result twice.
+        uint32_t a = v, b = v;
+        if constexpr (OFFSET == 16) asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+        else asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+        return {a, b};
+    }
+}
+template <int OFFSET>
+__device__ __forceinline__ float lane_xor_add(float v) {
+    const LanePair p = lane_xor_pair<OFFSET>(__builtin_bit_cast(uint32_t, v));
+    return __builtin_bit_cast(float, p.a) + __builtin_bit_cast(float, p.b);
+}
+template <int OFFSET>
+__device__ __forceinline__ float lane_xor_max(float v) {
+    const LanePair p = lane_xor_pair<OFFSET>(__builtin_bit_cast(uint32_t, v));
+    return fmaxf(__builtin_bit_cast(float, p.a), __builtin_bit_cast(float, p.b));
+}
+
 template <int FROM = 1, int TO = 64>
 __device__ __forceinline__ float lane_tree_sum(float v) {
-#pragma unroll
-    for (int o = FROM; o < TO; o <<= 1) v = v + __shfl_xor(v, o);
+    if constexpr (FROM <= 1 && TO > 1) v = lane_xor_add<1>(v);
+    if constexpr (FROM <= 2 && TO > 2) v = lane_xor_add<2>(v);
+    if constexpr (FROM <= 4 && TO > 4) v = lane_xor_add<4>(v);
+    if constexpr (FROM <= 8 && TO > 8) v = lane_xor_add<8>(v);
+    if constexpr (FROM <= 16 && TO > 16) v = lane_xor_add<16>(v);
+    if constexpr (FROM <= 32 && TO > 32) v = lane_xor_add<32>(v);
     return v;
 }
 template <int FROM = 1, int TO = 64>
 __device__ __forceinline__ float lane_tree_max(float v) {
-#pragma unroll
-    for (int o = FROM; o < TO; o <<= 1) v = fmaxf(v, __shfl_xor(v, o));
+    if constexpr (FROM <= 1 && TO > 1) v = lane_xor_max<1>(v);
+    if constexpr (FROM <= 2 && TO > 2) v = lane_xor_max<2>(v);
+    if constexpr (FROM <= 4 && TO > 4) v = lane_xor_max<4>(v);
+    if constexpr (FROM <= 8 && TO > 8) v = lane_xor_max<8>(v);
+    if constexpr (FROM <= 16 && TO > 16) v = lane_xor_max<16>(v);
+    if constexpr (FROM <= 32 && TO > 32) v = lane_xor_max<32>(v);
     return v;
 }
+template <int OFFSET>
+__device__ __forceinline__ int lane_xor_add_i32(int v) {
+    const LanePair p = lane_xor_pair<OFFSET>((uint32_t)v);
+    return (int)p.a + (int)p.b;
+}
 __device__ __forceinline__ int lane_sum_i32(int v) {
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) v += __shfl_xor(v, o);
+    v = lane_xor_add_i32<1>(v);
+    v = lane_xor_add_i32<2>(v);
+    v = lane_xor_add_i32<4>(v);
+    v = lane_xor_add_i32<8>(v);
+    v = lane_xor_add_i32<16>(v);
+    v = lane_xor_add_i32<32>(v);
+    return v;
+}
+
+// value of another lane through the DPP data path (no LDS round trip); lanes of rows not selected
+// by ROW_MASK read 0
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp_read(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false));
+}
+constexpr int kDppXor1 = 0xB1;         // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;         // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;  // lane i <- 7 - i within 8: the other quad once quads are uniform
+constexpr int kDppMirror = 0x140;      // lane i <- 15 - i within 16: the other half once halves are uniform
+constexpr int kDppBcast15 = 0x142;     // lane 15 of each row -> next row
+constexpr int kDppBcast31 = 0x143;     // lane 31 -> rows 2 and 3
+
+// Sum over the 64 lanes in the canonical tree order; the result is valid in lane 63 (returned as a
+// wave-uniform value).  Levels 1..8 are butterflies inside a row of 16; level 16 adds row 0 into
+// row 1 and row 2 into row 3; level 32 adds row 1 into row 3: ((r0+r1)+(r2+r3)).
+__device__ __forceinline__ float wave_tree_sum_uniform(float v) {
+    v = v + dpp_read<kDppXor1>(v);
+    v = v + dpp_read<kDppXor2>(v);
+    v = v + dpp_read<kDppHalfMirror>(v);
+    v = v + dpp_read<kDppMirror>(v);
+    v = v + dpp_read<kDppBcast15, 0xa>(v);
+    v = v + dpp_read<kDppBcast31, 0xc>(v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+// Sum over each aligned group of N lanes (N = 8 or 16), canonical order, valid in every lane.
+template <int N>
+__device__ __forceinline__ float group_tree_sum(float v) {
+    v = v + dpp_read<kDppXor1>(v);
+    v = v + dpp_read<kDppXor2>(v);
+    v = v + dpp_read<kDppHalfMirror>(v);
+    if (N == 16) v = v + dpp_read<kDppMirror>(v);
     return v;
 }
 
@@ -150,10 +270,22 @@ struct Ctx {
     int *arrive_o, *arrive_d;
     float *partial;
     int tid, wave, lane;
+    bool controller;
     int worker, slot, opcode;
     long long spin_ticks;           // wall-clock ticks (100 MHz) a wait may take
     int barrier_cols;               // H + 2 KVH
+    int *trace;                     // this instruction's timing row, or nullptr when tracing is off
+    long long t_launch;             // wall clock when the workgroup started
 };
+
+// Timing slots written per instruction by the controller when MK_FLAG_TIMINGS is set (ticks of
+// the 100 MHz wall clock since the workgroup started; counterpart of the reference's timing
+// events, include/util.cuh:215-246).
+enum { kEvStart = 0, kEvDepReady = 1, kEvInputReady = 2, kEvComputeDone = 3, kEvEnd = 4, kEvOpcode = 5 };
+
+__device__ __forceinline__ void trace_event(const Ctx &c, int slot) {
+    if (c.trace && c.controller && c.lane == 0) c.trace[slot] = (int)(wall_clock64() - c.t_launch);
+}
 
 __device__ __forceinline__ int *bar_ptr(const Ctx &c, int layer, int row, int col) {
     return c.a.barriers + ((size_t)layer * MK_BARRIER_ROWS + row) * c.barrier_cols + col;
@@ -172,63 +304,46 @@ __device__ void record_status(const Ctx &c, int code) {
     }
 }
 
-// Executed by all lanes of wave 0.  `ptr` is this lane's counter or nullptr.  sum_mode: wait until
-// the sum over lanes reaches target (sharded counter + its base value); otherwise wait until every
-// lane's counter reaches target.  Lane 63 watches the global status word so that one worker's
-// failure releases everybody.
-__device__ bool poll_wave0(const Ctx &c, const int *ptr, bool sum_mode, int target) {
+// Executed by all lanes of the controller wave.  `ptr` is this lane's counter or nullptr.
+// sum_mode: wait until the sum over lanes reaches target (sharded counter + its base value);
+// otherwise wait until every lane's counter reaches target.  Lane 63 watches the global status
+// word so that one worker's failure releases everybody.
+__device__ bool poll_counters(const Ctx &c, const int *ptr, bool sum_mode, int target) {
     const long long t0 = wall_clock64();
     while (true) {
         const int v = ptr ? ld_i32(ptr) : 0;
         const int st = c.lane == 63 ? ld_i32(c.status) : 0;
         const bool ok = sum_mode ? (lane_sum_i32(v) >= target) : (bool)__all(ptr == nullptr || v >= target);
-        if (ok) return true;
+        if (ok) break;
         if (__any(st != 0)) return false;
         if (wall_clock64() - t0 > c.spin_ticks) {
             if (c.lane == 0) record_status(c, MK_STATUS_BARRIER_TIMEOUT);
             return false;
         }
-        __builtin_amdgcn_s_sleep(2);
+        __builtin_amdgcn_s_sleep(1);
     }
+    compiler_fence();  // data loads stay after the successful poll
+    return true;
 }
 
-// Every instruction starts here: wave 0 waits for the dependency, then one workgroup barrier
-// publishes the outcome.  The barrier also separates the previous instruction's epilogue reads of
-// LDS from this instruction's writes.  Returns false when the launch is being abandoned.
-template <class Poll>
-__device__ __forceinline__ bool wait_dependency(const Ctx &c, Poll poll) {
-    if (c.wave == 0) {
-        if (!poll()) c.sm->abort = 1;
-    }
-    __syncthreads();
-    return c.sm->abort == 0;
+__device__ __forceinline__ bool poll_sharded(const Ctx &c, int layer, int row, int target) {
+    const int *p = nullptr;
+    if (c.lane < kShards) p = shard_ptr(c, c.lane, layer, row);
+    else if (c.lane == kShards) p = bar_ptr(c, layer, row, 0);
+    return poll_counters(c, p, true, target);
 }
 
-__device__ __forceinline__ bool wait_sharded(const Ctx &c, int layer, int row, int target) {
-    return wait_dependency(c, [&]() {
-        const int *p = nullptr;
-        if (c.lane < kShards) p = shard_ptr(c, c.lane, layer, row);
-        else if (c.lane == kShards) p = bar_ptr(c, layer, row, 0);
-        return poll_wave0(c, p, true, target);
-    });
-}
-__device__ __forceinline__ bool wait_nothing(const Ctx &c) {
-    return wait_dependency(c, [&]() { return true; });
-}
-// malformed instruction: record it and abandon the launch (all threads of the workgroup call this)
-__device__ __forceinline__ bool bail(const Ctx &c, int code) {
-    if (c.tid == 0) {
-        record_status(c, code);
-        c.sm->abort = 1;
-    }
-    __syncthreads();
-    return false;
-}
-
-// one arrival on a sharded counter; call from ONE thread after a __syncthreads that followed
-// the stores being published
+// one arrival on a sharded counter; the caller has waited for its stores
 __device__ __forceinline__ void signal_sharded(const Ctx &c, int layer, int row, int count) {
-    add_i32(shard_ptr(c, c.worker & (kShards - 1), layer, row), count);
+    if (c.lane == 0) add_i32(shard_ptr(c, c.worker & (kShards - 1), layer, row), count);
+}
+
+// Controller: publish the outcome of the dependency wait; everybody: first barrier of the
+// instruction.  Returns false when the launch is being abandoned.
+__device__ __forceinline__ bool barrier_inputs_ready(const Ctx &c, bool controller_ok) {
+    if (c.controller && !controller_ok && c.lane == 0) c.sm->abort = 1;
+    wg_barrier();
+    return c.sm->abort == 0;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -256,22 +371,17 @@ __device__ __forceinline__ void load_x(XVec<KC> &x, const uint16_t *src, int lan
     for (int j = 0; j < KC; j++) unpack8(raw[j], x.v[j]);
 }
 
-// python_vm.py:50-56: w * bf16(x * rsqrt(mean(x^2) + eps)), statistics in fp32.  Every wave
-// computes the whole vector for itself (4-8 KB from the memory-side cache), so no LDS and no
-// workgroup barrier are involved.
+// python_vm.py:50-56: w * bf16(x * rsqrt(mean(x^2) + eps)), statistics in fp32
 template <int KC>
-__device__ __forceinline__ void rms_norm_x(XVec<KC> &x, const uint16_t *hidden, const uint16_t *weight, float eps,
+__device__ __forceinline__ void rms_norm_x(XVec<KC> &x, const uint16_t *hidden, const uint4 (&wraw)[KC], float eps,
                                            int lane) {
-    uint4 wraw[KC];
-#pragma unroll
-    for (int j = 0; j < KC; j++) wraw[j] = ld_const_b128(weight + j * 512 + lane * 8);
     load_x<KC>(x, hidden, lane);
     float acc = 0.0f;
 #pragma unroll
     for (int j = 0; j < KC; j++)
 #pragma unroll
         for (int e = 0; e < 8; e++) acc = fmaf(x.v[j][e], x.v[j][e], acc);
-    const float mean = lane_tree_sum(acc) / (float)(KC * 512);
+    const float mean = wave_tree_sum_uniform(acc) / (float)(KC * 512);
     const float inv = 1.0f / sqrtf(mean + eps);
 #pragma unroll
     for (int j = 0; j < KC; j++) {
@@ -279,6 +389,27 @@ __device__ __forceinline__ void rms_norm_x(XVec<KC> &x, const uint16_t *hidden, 
         unpack8(wraw[j], wv);
 #pragma unroll
         for (int e = 0; e < 8; e++) x.v[j][e] = mkm::round_bf16(wv[e] * mkm::round_bf16(x.v[j][e] * inv));
+    }
+}
+
+// controller -> consumers hand-over of the activation vector, lane layout
+template <int KC>
+__device__ __forceinline__ void x_to_lds(const XVec<KC> &x, Smem *sm, int lane) {
+#pragma unroll
+    for (int j = 0; j < KC; j++) {
+        float4 *dst = reinterpret_cast<float4 *>(sm->x + (j * 64 + lane) * 8);
+        dst[0] = make_float4(x.v[j][0], x.v[j][1], x.v[j][2], x.v[j][3]);
+        dst[1] = make_float4(x.v[j][4], x.v[j][5], x.v[j][6], x.v[j][7]);
+    }
+}
+template <int KC>
+__device__ __forceinline__ void x_from_lds(XVec<KC> &x, const Smem *sm, int lane) {
+#pragma unroll
+    for (int j = 0; j < KC; j++) {
+        const float4 *src = reinterpret_cast<const float4 *>(sm->x + (j * 64 + lane) * 8);
+        const float4 lo = src[0], hi = src[1];
+        x.v[j][0] = lo.x; x.v[j][1] = lo.y; x.v[j][2] = lo.z; x.v[j][3] = lo.w;
+        x.v[j][4] = hi.x; x.v[j][5] = hi.y; x.v[j][6] = hi.z; x.v[j][7] = hi.w;
     }
 }
 
@@ -302,34 +433,55 @@ __device__ __forceinline__ float dot_row(const uint4 (&w)[KC], const XVec<KC> &x
         acc = fmaf(mkm::bf16_lo(w[j].w), x.v[j][6], acc);
         acc = fmaf(mkm::bf16_hi(w[j].w), x.v[j][7], acc);
     }
-    return lane_tree_sum(acc);
+    return wave_tree_sum_uniform(acc);
 }
 
-// Streams `ntasks` weight rows through the workgroup: task t is handled by wave t % 16 and its
-// bf16-rounded dot product lands in sm->out[t].  PF rows per wave are in flight; the first PF are
-// requested before `wait` (the dependency) and `make_x` (the activation vector) run.
-template <int KC, int PF, class RowPtr, class Wait, class MakeX>
-__device__ __forceinline__ bool stream_rows(const Ctx &c, int ntasks, RowPtr row_ptr, Wait wait, MakeX make_x) {
-    const int mine = ntasks > c.wave ? (ntasks - c.wave + kWaves - 1) / kWaves : 0;
+// One batch of a matvec instruction.
+//   consumers : request the first rows, barrier (activation vector ready), stream `ntasks` rows
+//               (task t -> wave t % 8, result bf16-rounded into sm->out[t]), barrier (results ready)
+//   controller: `prepare` (wait for the dependency, build the activation vector in LDS; returns
+//               false to abandon), barrier, barrier, `finish` (epilogue + signal)
+// Both barriers are reached by all nine waves whatever the outcome of `prepare`.
+template <int KC, class RowPtr, class Prepare, class Finish>
+__device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need_x, RowPtr row_ptr, Prepare prepare,
+                                             Finish finish) {
+    constexpr int PF = rows_in_flight<KC>();
+    if (c.controller) {
+        const bool ok = prepare();
+        trace_event(c, kEvInputReady);
+        if (!barrier_inputs_ready(c, ok)) return false;
+        wg_barrier();
+        trace_event(c, kEvComputeDone);
+        finish();
+        return true;
+    }
+    const int mine = ntasks > c.wave ? (ntasks - c.wave + kConsumerWaves - 1) / kConsumerWaves : 0;
     uint4 buf[PF][KC];
 #pragma unroll
     for (int s = 0; s < PF; s++)
-        if (s < mine) load_row<KC>(buf[s], row_ptr(c.wave + s * kWaves), c.lane);
-    if (!wait()) return false;
+        if (s < mine) load_row<KC>(buf[s], row_ptr(c.wave + s * kConsumerWaves), c.lane);
+    if (!barrier_inputs_ready(c, true)) return false;
     XVec<KC> x;
-    make_x(x);
+    if (need_x) x_from_lds<KC>(x, c.sm, c.lane);
     for (int base = 0; base < mine; base += PF) {
 #pragma unroll
         for (int s = 0; s < PF; s++) {
             const int i = base + s;
             if (i < mine) {
                 const float y = mkm::round_bf16(dot_row<KC>(buf[s], x));
-                if (i + PF < mine) load_row<KC>(buf[s], row_ptr(c.wave + (i + PF) * kWaves), c.lane);
-                if (c.lane == 0) c.sm->out[c.wave + i * kWaves] = y;
+                if (i + PF < mine) load_row<KC>(buf[s], row_ptr(c.wave + (i + PF) * kConsumerWaves), c.lane);
+                if (c.lane == 0) c.sm->out[c.wave + i * kConsumerWaves] = y;
             }
         }
     }
+    wg_barrier();
     return true;
+}
+
+// malformed instruction: every wave evaluates the same condition and leaves; the controller records it
+__device__ __forceinline__ bool bail(const Ctx &c, int code) {
+    if (c.controller && c.lane == 0) record_status(c, code);
+    return false;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -337,56 +489,60 @@ __device__ __forceinline__ bool stream_rows(const Ctx &c, int ntasks, RowPtr row
 // reference device op: demos/low-latency-llama/rms_matvec_rope_append.cu:10-231)
 // ---------------------------------------------------------------------------------------------
 template <int KC>
-__device__ bool op_qkv(const Ctx &c, const int *ins) {
+__device__ __forceinline__ bool op_qkv(const Ctx &c, const int *ins) {
     const mk_llama_args &a = c.a;
     const int layer = ins[1], start = ins[2], end = ins[3];
     const int hid = a.hidden_size, D = a.head_dim, H = a.num_attention_heads, KVH = a.num_kv_heads;
     const int total_blocks = (H + 2 * KVH) * D / 16;
-    if (layer < 0 || layer >= a.num_layers || start < 0 || end > total_blocks || end - start > kOutRows / 16) return bail(c, MK_STATUS_BAD_INSTRUCTION);
+    if (layer < 0 || layer >= a.num_layers || start < 0 || end > total_blocks || end - start > kOutRows / 16)
+        return bail(c, MK_STATUS_BAD_INSTRUCTION);
     const int nblk = end > start ? end - start : 0;
     const uint16_t *W = a.qkv_weights + (size_t)layer * total_blocks * 16 * hid;
     const int down_jobs = (a.intermediate_size / a.matvec_reduction_size) * (hid / 16);
 
-    const bool ok = stream_rows<KC, rows_in_flight<KC>(2)>(
-        c, nblk * 16, [&](int t) { return W + (size_t)(start * 16 + t) * hid; },
-        [&]() { return layer > 0 ? wait_sharded(c, layer - 1, 5, down_jobs) : wait_nothing(c); },
-        [&](XVec<KC> &x) {
-            if (nblk > 0)
-                rms_norm_x<KC>(x, a.hidden_states, a.attn_norm_weights + (size_t)layer * hid, a.rms_norm_eps, c.lane);
+    return matvec_batch<KC>(
+        c, nblk * 16, nblk > 0, [&](int t) { return W + (size_t)(start * 16 + t) * hid; },
+        [&]() {
+            uint4 wraw[KC];
+            if (nblk > 0) load_row<KC>(wraw, a.attn_norm_weights + (size_t)layer * hid, c.lane);
+            if (layer > 0 && !poll_sharded(c, layer - 1, 5, down_jobs)) return false;
+            trace_event(c, kEvDepReady);
+            if (nblk > 0) {
+                XVec<KC> x;
+                rms_norm_x<KC>(x, a.hidden_states, wraw, a.rms_norm_eps, c.lane);
+                x_to_lds<KC>(x, c.sm, c.lane);
+            }
+            return true;
+        },
+        [&]() {
+            // epilogue: one lane per adjacent row pair
+            const int k_start = H * D, v_start = k_start + KVH * D;
+            const size_t kv_row = ((size_t)layer * a.kv_max_len + a.pos_id) * KVH * D;
+            for (int p = c.lane; p < nblk * 8; p += 64) {
+                const int row0 = start * 16 + p * 2;
+                const float y0 = c.sm->out[p * 2], y1 = c.sm->out[p * 2 + 1];
+                uint32_t packed;
+                if (row0 < v_start) {
+                    // interleaved rotary embedding (llama.py:136-174): products and sum in fp32, unfused
+                    const int d = row0 % D;
+                    const float *cs = a.rope_cos + (size_t)a.pos_id * D + d;
+                    const float *sn = a.rope_sin + (size_t)a.pos_id * D + d;
+                    const float even = (y0 * cs[0]) + ((-y1) * sn[0]);
+                    const float odd = (y1 * cs[1]) + (y0 * sn[1]);
+                    packed = mkm::pack_bf16(even, odd);
+                } else {
+                    packed = mkm::pack_bf16(y0, y1);
+                }
+                uint16_t *dst;
+                if (row0 < k_start) dst = a.q_post_rope + row0;
+                else if (row0 < v_start) dst = a.k_cache + kv_row + (row0 - k_start);
+                else dst = a.v_cache + kv_row + (row0 - v_start);
+                st_u32(dst, packed);
+            }
+            wait_stores();
+            // one arrival per block on its head's counter (python_vm.py:248)
+            for (int b = c.lane; b < nblk; b += 64) add_i32(bar_ptr(c, layer, 0, (start + b) / (D / 16)), 1);
         });
-    if (!ok) return false;
-    if (nblk == 0) return true;
-    __syncthreads();
-
-    // epilogue: one thread per adjacent row pair
-    const int k_start = H * D, v_start = k_start + KVH * D;
-    if (c.tid < nblk * 8) {
-        const int lb = c.tid >> 3, pair = c.tid & 7;
-        const int row0 = (start + lb) * 16 + pair * 2;
-        const float y0 = c.sm->out[lb * 16 + pair * 2], y1 = c.sm->out[lb * 16 + pair * 2 + 1];
-        uint32_t packed;
-        if (row0 < v_start) {
-            // interleaved rotary embedding (llama.py:136-174): products and sum in fp32, unfused
-            const int d = row0 % D;
-            const float *cs = a.rope_cos + (size_t)a.pos_id * D + d;
-            const float *sn = a.rope_sin + (size_t)a.pos_id * D + d;
-            const float even = (y0 * cs[0]) + ((-y1) * sn[0]);
-            const float odd = (y1 * cs[1]) + (y0 * sn[1]);
-            packed = mkm::pack_bf16(even, odd);
-        } else {
-            packed = mkm::pack_bf16(y0, y1);
-        }
-        uint16_t *dst;
-        const size_t kv_row = ((size_t)layer * a.kv_max_len + a.pos_id) * KVH * D;
-        if (row0 < k_start) dst = a.q_post_rope + row0;
-        else if (row0 < v_start) dst = a.k_cache + kv_row + (row0 - k_start);
-        else dst = a.v_cache + kv_row + (row0 - v_start);
-        st_u32(dst, packed);
-    }
-    __syncthreads();
-    // one arrival per block on the head's counter (python_vm.py:248)
-    if (c.tid < nblk) add_i32(bar_ptr(c, layer, 0, (start + c.tid) / (D / 16)), 1);
-    return true;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -398,66 +554,71 @@ __device__ bool op_qkv(const Ctx &c, const int *ins) {
 // rounding chain is reproduced without serialising the workers.
 // ---------------------------------------------------------------------------------------------
 template <int KC>
-__device__ bool op_matvec_add(const Ctx &c, const int *ins, bool is_down) {
+__device__ __forceinline__ bool op_matvec_add(const Ctx &c, const int *ins, bool is_down) {
     const mk_llama_args &a = c.a;
     const int layer = ins[1], start = ins[2], end = ins[3], group = ins[4];
     const int hid = a.hidden_size, R = a.matvec_reduction_size;
     const int in_dim = is_down ? a.intermediate_size : hid;
     const int ngroups = in_dim / R;
     if (layer < 0 || layer >= a.num_layers || start < 0 || end > hid / 16 || group < 0 || group >= ngroups ||
-        end - start > kOutRows / 16) return bail(c, MK_STATUS_BAD_INSTRUCTION);
+        end - start > kOutRows / 16)
+        return bail(c, MK_STATUS_BAD_INSTRUCTION);
     const int nblk = end > start ? end - start : 0;
     const uint16_t *W = (is_down ? a.down_weights : a.o_weights) + (size_t)layer * hid * in_dim + (size_t)group * R;
     const uint16_t *vec = (is_down ? a.silu_out : a.attn_out) + (size_t)group * R;
     const int wait_row = is_down ? 4 : 2;
     const int wait_target = is_down ? a.intermediate_size / 16 : a.num_attention_heads;
-
-    const bool ok = stream_rows<KC, rows_in_flight<KC>(2)>(
-        c, nblk * 16, [&](int t) { return W + (size_t)(start * 16 + t) * in_dim; },
-        [&]() { return wait_sharded(c, layer, wait_row, wait_target); },
-        [&](XVec<KC> &x) {
-            if (nblk > 0) load_x<KC>(x, vec, c.lane);
-        });
-    if (!ok) return false;
-    if (nblk == 0) return true;
-    __syncthreads();
-
     uint16_t *resid = a.hidden_states;
-    if (ngroups == 1) {
-        if (c.tid < nblk * 8) {
-            const int t0 = c.tid * 2;
-            const int row0 = start * 16 + t0;
-            const uint32_t h = ld_u32(resid + row0);
-            const float lo = mkm::bf16_lo(h) + c.sm->out[t0];
-            const float hi = mkm::bf16_hi(h) + c.sm->out[t0 + 1];
-            st_u32(resid + row0, mkm::pack_bf16(lo, hi));
-        }
-    } else {
-        int *arrive = is_down ? c.arrive_d : c.arrive_o;
-        if (c.tid < nblk * 16) st_f32(c.partial + (size_t)group * hid + start * 16 + c.tid, c.sm->out[c.tid]);
-        __syncthreads();
-        if (c.tid < nblk) {
-            const int old = __hip_atomic_fetch_add(&arrive[start + c.tid], 1, __ATOMIC_RELAXED, AG);
-            const int last = old == ngroups - 1;
-            if (last) st_i32(&arrive[start + c.tid], 0);
-            c.sm->flags[c.tid] = last;
-        }
-        __syncthreads();
-        if (c.tid < nblk * 8 && c.sm->flags[c.tid >> 3]) {
-            const int row0 = start * 16 + c.tid * 2;
-            const uint32_t h = ld_u32(resid + row0);
-            float lo = mkm::bf16_lo(h), hi = mkm::bf16_hi(h);
-            for (int g = 0; g < ngroups; g++) {
-                const uint64_t p = ld_u64(c.partial + (size_t)g * hid + row0);
-                lo = mkm::round_bf16(lo + mkm::bits_f32((uint32_t)p));
-                hi = mkm::round_bf16(hi + mkm::bits_f32((uint32_t)(p >> 32)));
+
+    return matvec_batch<KC>(
+        c, nblk * 16, nblk > 0, [&](int t) { return W + (size_t)(start * 16 + t) * in_dim; },
+        [&]() {
+            if (!poll_sharded(c, layer, wait_row, wait_target)) return false;
+            trace_event(c, kEvDepReady);
+            if (nblk > 0) {
+                XVec<KC> x;
+                load_x<KC>(x, vec, c.lane);
+                x_to_lds<KC>(x, c.sm, c.lane);
             }
-            st_u32(resid + row0, mkm::pack_bf16(lo, hi));
-        }
-    }
-    __syncthreads();
-    if (c.tid == 0) signal_sharded(c, layer, is_down ? 5 : 3, nblk);
-    return true;
+            return true;
+        },
+        [&]() {
+            if (ngroups == 1) {
+                for (int p = c.lane; p < nblk * 8; p += 64) {
+                    const int row0 = start * 16 + p * 2;
+                    const uint32_t h = ld_u32(resid + row0);
+                    const float lo = mkm::bf16_lo(h) + c.sm->out[p * 2];
+                    const float hi = mkm::bf16_hi(h) + c.sm->out[p * 2 + 1];
+                    st_u32(resid + row0, mkm::pack_bf16(lo, hi));
+                }
+            } else {
+                int *arrive = is_down ? c.arrive_d : c.arrive_o;
+                for (int t = c.lane; t < nblk * 16; t += 64)
+                    st_f32(c.partial + (size_t)group * hid + start * 16 + t, c.sm->out[t]);
+                wait_stores();
+                for (int b = c.lane; b < nblk; b += 64) {
+                    const int old = __hip_atomic_fetch_add(&arrive[start + b], 1, __ATOMIC_RELAXED, AG);
+                    const int last = old == ngroups - 1;
+                    if (last) st_i32(&arrive[start + b], 0);
+                    c.sm->flags[b] = last;
+                }
+                compiler_fence();  // same wave: LDS operations execute in order
+                for (int p = c.lane; p < nblk * 8; p += 64) {
+                    if (!c.sm->flags[p >> 3]) continue;
+                    const int row0 = start * 16 + p * 2;
+                    const uint32_t h = ld_u32(resid + row0);
+                    float lo = mkm::bf16_lo(h), hi = mkm::bf16_hi(h);
+                    for (int g = 0; g < ngroups; g++) {
+                        const uint64_t v = ld_u64(c.partial + (size_t)g * hid + row0);
+                        lo = mkm::round_bf16(lo + mkm::bits_f32((uint32_t)v));
+                        hi = mkm::round_bf16(hi + mkm::bits_f32((uint32_t)(v >> 32)));
+                    }
+                    st_u32(resid + row0, mkm::pack_bf16(lo, hi));
+                }
+            }
+            wait_stores();
+            signal_sharded(c, layer, is_down ? 5 : 3, nblk);
+        });
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -465,7 +626,7 @@ __device__ bool op_matvec_add(const Ctx &c, const int *ins, bool is_down) {
 // reference device op: demos/low-latency-llama/upgate.cu:10-172)
 // ---------------------------------------------------------------------------------------------
 template <int KC>
-__device__ bool op_upgate(const Ctx &c, const int *ins) {
+__device__ __forceinline__ bool op_upgate(const Ctx &c, const int *ins) {
     const mk_llama_args &a = c.a;
     const int layer = ins[1], n = ins[2];
     const int hid = a.hidden_size, inter = a.intermediate_size;
@@ -478,32 +639,36 @@ __device__ bool op_upgate(const Ctx &c, const int *ins) {
     const int o_jobs = (hid / a.matvec_reduction_size) * (hid / 16);
 
     // task t: list entry t / 32, matrix (t / 16) & 1 (0 up, 1 gate), row t % 16
-    const bool ok = stream_rows<KC, rows_in_flight<KC>(4)>(
-        c, n * 32,
+    return matvec_batch<KC>(
+        c, n * 32, n > 0,
         [&](int t) {
             const int blk = ins[3 + (t >> 5)];
             return ((t >> 4) & 1 ? Wg : Wu) + (size_t)(blk * 16 + (t & 15)) * hid;
         },
-        [&]() { return wait_sharded(c, layer, 3, o_jobs); },
-        [&](XVec<KC> &x) {
-            if (n > 0)
-                rms_norm_x<KC>(x, a.hidden_states, a.mlp_norm_weights + (size_t)layer * hid, a.rms_norm_eps, c.lane);
+        [&]() {
+            uint4 wraw[KC];
+            if (n > 0) load_row<KC>(wraw, a.mlp_norm_weights + (size_t)layer * hid, c.lane);
+            if (!poll_sharded(c, layer, 3, o_jobs)) return false;
+            trace_event(c, kEvDepReady);
+            if (n > 0) {
+                XVec<KC> x;
+                rms_norm_x<KC>(x, a.hidden_states, wraw, a.rms_norm_eps, c.lane);
+                x_to_lds<KC>(x, c.sm, c.lane);
+            }
+            return true;
+        },
+        [&]() {
+            for (int p = c.lane; p < n * 8; p += 64) {
+                const int i = p >> 3, r = (p & 7) * 2;
+                const float *up = c.sm->out + i * 32, *gate = up + 16;
+                // silu(gate) -> bf16, then times up -> bf16 (python_vm.py:161-163)
+                const float s0 = mkm::round_bf16(mkm::silu_exact(gate[r]));
+                const float s1 = mkm::round_bf16(mkm::silu_exact(gate[r + 1]));
+                st_u32(a.silu_out + ins[3 + i] * 16 + r, mkm::pack_bf16(s0 * up[r], s1 * up[r + 1]));
+            }
+            wait_stores();
+            signal_sharded(c, layer, 4, n);
         });
-    if (!ok) return false;
-    if (n == 0) return true;
-    __syncthreads();
-    if (c.tid < n * 8) {
-        const int i = c.tid >> 3, pair = c.tid & 7;
-        const float *up = c.sm->out + i * 32, *gate = up + 16;
-        const int r = pair * 2;
-        // silu(gate) -> bf16, then times up -> bf16 (python_vm.py:161-163)
-        const float s0 = mkm::round_bf16(mkm::silu_exact(gate[r]));
-        const float s1 = mkm::round_bf16(mkm::silu_exact(gate[r + 1]));
-        st_u32(a.silu_out + ins[3 + i] * 16 + r, mkm::pack_bf16(s0 * up[r], s1 * up[r + 1]));
-    }
-    __syncthreads();
-    if (c.tid == 0) signal_sharded(c, layer, 4, n);
-    return true;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -511,7 +676,7 @@ __device__ bool op_upgate(const Ctx &c, const int *ins) {
 // reference device op: demos/low-latency-llama/rms_lm_head.cu:10-117)
 // ---------------------------------------------------------------------------------------------
 template <int KC>
-__device__ bool op_lm_head(const Ctx &c, const int *ins) {
+__device__ __forceinline__ bool op_lm_head(const Ctx &c, const int *ins) {
     const mk_llama_args &a = c.a;
     const int start = ins[1], end = ins[2];
     const int hid = a.hidden_size;
@@ -523,16 +688,24 @@ __device__ bool op_lm_head(const Ctx &c, const int *ins) {
     do {
         const int b1 = min(b0 + blocks_per_batch, end);
         const int nblk = b1 > b0 ? b1 - b0 : 0;
-        const bool ok = stream_rows<KC, rows_in_flight<KC>(4)>(
-            c, nblk * 16, [&](int t) { return a.lm_head_weights + (size_t)(b0 * 16 + t) * hid; },
-            [&]() { return first ? wait_sharded(c, a.num_layers - 1, 5, down_jobs) : wait_nothing(c); },
-            [&](XVec<KC> &x) {
-                if (nblk > 0) rms_norm_x<KC>(x, a.hidden_states, a.lm_head_norm_weights, a.rms_norm_eps, c.lane);
+        const bool ok = matvec_batch<KC>(
+            c, nblk * 16, true, [&](int t) { return a.lm_head_weights + (size_t)(b0 * 16 + t) * hid; },
+            [&]() {
+                if (!first) return true;  // the activation vector stays in LDS between batches
+                uint4 wraw[KC];
+                load_row<KC>(wraw, a.lm_head_norm_weights, c.lane);
+                if (!poll_sharded(c, a.num_layers - 1, 5, down_jobs)) return false;
+                trace_event(c, kEvDepReady);
+                XVec<KC> x;
+                rms_norm_x<KC>(x, a.hidden_states, wraw, a.rms_norm_eps, c.lane);
+                x_to_lds<KC>(x, c.sm, c.lane);
+                return true;
+            },
+            [&]() {
+                for (int p = c.lane; p < nblk * 8; p += 64)
+                    st_u32(a.logits + b0 * 16 + p * 2, mkm::pack_bf16(c.sm->out[p * 2], c.sm->out[p * 2 + 1]));
             });
         if (!ok) return false;
-        __syncthreads();
-        for (int p = c.tid; p < nblk * 8; p += kThreads)
-            st_u32(a.logits + b0 * 16 + p * 2, mkm::pack_bf16(c.sm->out[p * 2], c.sm->out[p * 2 + 1]));
         first = false;
         b0 = b1;
     } while (b0 < end);
@@ -540,26 +713,29 @@ __device__ bool op_lm_head(const Ctx &c, const int *ins) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// opcode 2: attention of the G query heads of one KV head over one partition of the cache
+// opcode 2: attention of the 4 query heads of one KV head over one partition of the cache
 // (python_vm.py:277-346; reference device op: demos/low-latency-llama/attention_partial.cu).
 // Two passes over LDS-resident scores: (1) s = scale * q.k for every token, exact maximum;
 // (2) p = exp(s - max), slot sums of p and p*v.  Token r of the partition belongs to slot
-// r mod NSLOT with NSLOT = 16 waves * (64 / (D/8)) tokens per wave load; a slot accumulates its
-// tokens in increasing order and slots are combined by a pairwise tree (lanes, then waves).
+// r mod NSLOT, NSLOT = 16 virtual waves * (64 / (D/8)) tokens per wave load; a slot accumulates
+// its tokens in increasing order and slots are combined by a pairwise tree (lanes, then virtual
+// waves).  Each of the 8 consumer waves plays virtual waves w and w + 8.
 // ---------------------------------------------------------------------------------------------
 template <int D>
-__device__ bool op_attention(const Ctx &c, const int *ins) {
-    constexpr int LPT = D / 8;            // lanes per token
-    constexpr int TPW = 64 / LPT;         // tokens per wave per round
-    constexpr int NSLOT = kWaves * TPW;   // tokens per workgroup round
-    constexpr int G = kGqaMax;
+__device__ __forceinline__ bool op_attention(const Ctx &c, const int *ins) {
+    constexpr int LPT = D / 8;                  // lanes per token
+    constexpr int TPW = 64 / LPT;               // tokens per wave per round
+    constexpr int NSLOT = kVirtualWaves * TPW;  // tokens per workgroup round
+    constexpr int G = kGqa;
+    constexpr int VW = kVirtualWaves / kConsumerWaves;  // virtual waves per consumer wave
     const mk_llama_args &a = c.a;
     Smem *sm = c.sm;
     const int layer = ins[1], kvh = ins[2], P = ins[3], pidx = ins[4];
     const int H = a.num_attention_heads, KVH = a.num_kv_heads;
     const bool skip = a.skip_attn_reduction != 0;
     if (layer < 0 || layer >= a.num_layers || kvh < 0 || kvh >= KVH || P < 1 || pidx < 0 || pidx >= P ||
-        (!skip && pidx >= a.max_partials)) return bail(c, MK_STATUS_BAD_INSTRUCTION);
+        (!skip && pidx >= a.max_partials))
+        return bail(c, MK_STATUS_BAD_INSTRUCTION);
     const int seq_len = a.pos_id + 1;
     const int total_blocks = (seq_len + 15) / 16;
     const int bpp = (total_blocks + P - 1) / P;
@@ -570,137 +746,178 @@ __device__ bool op_attention(const Ctx &c, const int *ins) {
     const int T = t1 > t0 ? t1 - t0 : 0;
     if (T > kScoreCap) return bail(c, MK_STATUS_ATTN_TOO_LONG);
     const int h0 = kvh * G;
-    const int sub = c.lane % LPT;         // which 8 dims of the head this lane owns
-    const int tok_in_wave = c.lane / LPT;
-    const int slot = c.wave * TPW + tok_in_wave;
-    const size_t tok_stride = (size_t)KVH * D;
-    const size_t base = ((size_t)layer * a.kv_max_len) * tok_stride + (size_t)kvh * D + sub * 8;
-    const uint16_t *kbase = a.k_cache + base;
-    const uint16_t *vbase = a.v_cache + base;
     const int rounds = (T + NSLOT - 1) / NSLOT;
 
-    // wait: Q heads, K head and V head of this step are complete (python_vm.py:281-290)
-    const int per_head = D / 16;
-    const bool ok = wait_dependency(c, [&]() {
+    if (c.controller) {
+        // wait: Q heads, K head and V head of this step are complete (python_vm.py:281-290)
         const int *p = nullptr;
         if (c.lane < G) p = bar_ptr(c, layer, 0, h0 + c.lane);
         else if (c.lane == G) p = bar_ptr(c, layer, 0, H + kvh);
         else if (c.lane == G + 1) p = bar_ptr(c, layer, 0, H + KVH + kvh);
-        return poll_wave0(c, p, false, per_head);
-    });
-    if (!ok) return false;
+        const bool ok = poll_counters(c, p, false, D / 16);
+        trace_event(c, kEvDepReady);
+        if (!barrier_inputs_ready(c, ok)) return false;
+        wg_barrier();  // wave maxima
+        trace_event(c, 6);
+        wg_barrier();  // probabilities
+        trace_event(c, 7);
+        wg_barrier();  // wave sums
+        trace_event(c, 8);
+        wg_barrier();  // outputs stored
+        trace_event(c, kEvComputeDone);
+        if (skip) signal_sharded(c, layer, 2, G);
+        else if (c.lane < G) add_i32(bar_ptr(c, layer, 1, h0 + c.lane), 1);
+        return true;
+    }
 
-    // token row loads: rows older than this step are immutable, the row at pos_id was written by
-    // another CU a moment ago and needs a coherent load
+    const int sub = c.lane % LPT;         // which 8 dims of the head this lane owns
+    const int tok_in_wave = c.lane / LPT;
+    const size_t tok_stride = (size_t)KVH * D;
+    const size_t base = ((size_t)layer * a.kv_max_len) * tok_stride + (size_t)kvh * D + sub * 8;
+    const uint16_t *kbase = a.k_cache + base;
+    const uint16_t *vbase = a.v_cache + base;
+    // relative token handled by this lane in round rd as virtual wave v
+    auto token_of = [&](int rd, int v) { return rd * NSLOT + (c.wave + v * kConsumerWaves) * TPW + tok_in_wave; };
+    // rows older than this step are immutable; the row at pos_id was written by another CU a moment
+    // ago and needs a coherent load
     auto load_kv = [&](const uint16_t *kvb, int r) {
         const int t = t0 + r;
         const uint16_t *p = kvb + (size_t)t * tok_stride;
         return t == a.pos_id ? ld_b128(p) : ld_const_b128(p);
     };
 
+    // round 0 of K does not depend on this step except for the newest token: request it early
+    uint4 k0[VW];
+#pragma unroll
+    for (int v = 0; v < VW; v++) {
+        const int r = token_of(0, v);
+        k0[v] = make_uint4(0, 0, 0, 0);
+        if (r < T && t0 + r != a.pos_id) k0[v] = ld_const_b128(kbase + (size_t)(t0 + r) * tok_stride);
+    }
+    if (!barrier_inputs_ready(c, true)) return false;
+
     float q[G][8];
 #pragma unroll
-    for (int h = 0; h < G; h++) {
-        float tmp[8];
-        unpack8(ld_b128(a.q_post_rope + (size_t)(h0 + h) * D + sub * 8), tmp);
-#pragma unroll
-        for (int e = 0; e < 8; e++) q[h][e] = tmp[e];
-    }
+    for (int h = 0; h < G; h++) unpack8(ld_b128(a.q_post_rope + (size_t)(h0 + h) * D + sub * 8), q[h]);
 
     // ---- pass 1: scores and maximum ----
-    float mx[G];
+    float mx[VW][G];
 #pragma unroll
-    for (int h = 0; h < G; h++) mx[h] = -INFINITY;
+    for (int v = 0; v < VW; v++)
+#pragma unroll
+        for (int h = 0; h < G; h++) mx[v][h] = -INFINITY;
     for (int rd = 0; rd < rounds; rd++) {
-        const int r = rd * NSLOT + slot;
-        if (r < T) {
-            float kf[8];
-            unpack8(load_kv(kbase, r), kf);
+        uint4 kraw[VW];
 #pragma unroll
-            for (int h = 0; h < G; h++) {
-                float acc = 0.0f;
+        for (int v = 0; v < VW; v++) {
+            const int r = token_of(rd, v);
+            kraw[v] = k0[v];
+            if (r < T && (rd > 0 || t0 + r == a.pos_id)) kraw[v] = load_kv(kbase, r);
+        }
 #pragma unroll
-                for (int e = 0; e < 8; e++) acc = fmaf(q[h][e], kf[e], acc);
-                // the LPT lanes of a token share r, so they are active together
-                const float s = lane_tree_sum<1, LPT>(acc) * a.attn_scale;
-                if (sub == 0) sm->scores[h][r] = s;
-                mx[h] = fmaxf(mx[h], s);
+        for (int v = 0; v < VW; v++) {
+            const int r = token_of(rd, v);
+            if (r < T) {  // the LPT lanes of a token share r, so they are active together
+                float kf[8];
+                unpack8(kraw[v], kf);
+#pragma unroll
+                for (int h = 0; h < G; h++) {
+                    float acc = 0.0f;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) acc = fmaf(q[h][e], kf[e], acc);
+                    const float s = group_tree_sum<LPT>(acc) * a.attn_scale;
+                    if (sub == 0) sm->scores[h][r] = s;
+                    mx[v][h] = fmaxf(mx[v][h], s);
+                }
             }
         }
     }
 #pragma unroll
-    for (int h = 0; h < G; h++) {
-        const float m = lane_tree_max<LPT, 64>(mx[h]);
-        if (c.lane == 0) sm->wave_max[c.wave][h] = m;
-    }
-    __syncthreads();
-    if (c.tid < G) {
-        float m = sm->wave_max[0][c.tid];
-        for (int w = 1; w < kWaves; w++) m = fmaxf(m, sm->wave_max[w][c.tid]);
-        sm->head_m[c.tid] = m;
-    }
-    __syncthreads();
-    // p = exp(s - max), once per (head, token), in place
-    for (int i = c.tid; i < G * T; i += kThreads) {
-        const int h = i / T, r = i - h * T;
-        sm->scores[h][r] = mkm::expf_exact(sm->scores[h][r] - sm->head_m[h]);
-    }
-    __syncthreads();
-
-    // ---- pass 2: slot sums ----
-    float acc[G][8], lsum[G];
-#pragma unroll
-    for (int h = 0; h < G; h++) {
-        lsum[h] = 0.0f;
-#pragma unroll
-        for (int e = 0; e < 8; e++) acc[h][e] = 0.0f;
-    }
-    for (int rd = 0; rd < rounds; rd++) {
-        const int r = rd * NSLOT + slot;
-        if (r < T) {
-            float vf[8];
-            unpack8(load_kv(vbase, r), vf);
-#pragma unroll
-            for (int h = 0; h < G; h++) {
-                const float p = sm->scores[h][r];
-                lsum[h] = lsum[h] + p;
-#pragma unroll
-                for (int e = 0; e < 8; e++) acc[h][e] = fmaf(p, vf[e], acc[h][e]);
-            }
-        }
-    }
-    // combine the TPW slots of this wave (pairwise tree over lane groups), then park per wave
-#pragma unroll
-    for (int h = 0; h < G; h++) {
-        lsum[h] = lane_tree_sum<LPT, 64>(lsum[h]);
-#pragma unroll
-        for (int e = 0; e < 8; e++) acc[h][e] = lane_tree_sum<LPT, 64>(acc[h][e]);
-    }
-    if (c.lane < LPT) {
+    for (int v = 0; v < VW; v++)
 #pragma unroll
         for (int h = 0; h < G; h++) {
+            const float m = lane_tree_max<LPT, 64>(mx[v][h]);
+            if (c.lane == 0) sm->wave_max[c.wave + v * kConsumerWaves][h] = m;
+        }
+    wg_barrier();
+    float hm[G];
 #pragma unroll
-            for (int e = 0; e < 8; e++) sm->wave_o[c.wave][h][sub * 8 + e] = acc[h][e];
-            if (c.lane == 0) sm->wave_l[c.wave][h] = lsum[h];
+    for (int h = 0; h < G; h++) {
+        float m = sm->wave_max[0][h];
+        for (int w = 1; w < kVirtualWaves; w++) m = fmaxf(m, sm->wave_max[w][h]);
+        hm[h] = m;
+    }
+    // p = exp(s - max), once per (head, token), in place
+    for (int i = c.tid; i < G * T; i += kConsumerThreads) {
+        const int h = i / T, r = i - h * T;
+        const float m = h == 0 ? hm[0] : h == 1 ? hm[1] : h == 2 ? hm[2] : hm[3];
+        sm->scores[h][r] = mkm::expf_exact(sm->scores[h][r] - m);
+    }
+    wg_barrier();
+
+    // ---- pass 2: slot sums ----
+    float acc[VW][G][8], lsum[VW][G];
+#pragma unroll
+    for (int v = 0; v < VW; v++)
+#pragma unroll
+        for (int h = 0; h < G; h++) {
+            lsum[v][h] = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc[v][h][e] = 0.0f;
+        }
+    for (int rd = 0; rd < rounds; rd++) {
+        uint4 vraw[VW];
+#pragma unroll
+        for (int v = 0; v < VW; v++) {
+            const int r = token_of(rd, v);
+            vraw[v] = make_uint4(0, 0, 0, 0);
+            if (r < T) vraw[v] = load_kv(vbase, r);
+        }
+#pragma unroll
+        for (int v = 0; v < VW; v++) {
+            const int r = token_of(rd, v);
+            if (r < T) {
+                float vf[8];
+                unpack8(vraw[v], vf);
+#pragma unroll
+                for (int h = 0; h < G; h++) {
+                    const float p = sm->scores[h][r];
+                    lsum[v][h] = lsum[v][h] + p;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) acc[v][h][e] = fmaf(p, vf[e], acc[v][h][e]);
+                }
+            }
         }
     }
-    __syncthreads();
+    // combine the TPW slots of each virtual wave (pairwise tree over lane groups), park per wave
+#pragma unroll
+    for (int v = 0; v < VW; v++)
+#pragma unroll
+        for (int h = 0; h < G; h++) {
+            const float l = lane_tree_sum<LPT, 64>(lsum[v][h]);
+            if (c.lane == 0) sm->wave_l[c.wave + v * kConsumerWaves][h] = l;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float o = lane_tree_sum<LPT, 64>(acc[v][h][e]);
+                if (c.lane < LPT) sm->wave_o[c.wave + v * kConsumerWaves][h][sub * 8 + e] = o;
+            }
+        }
+    wg_barrier();
 
-    // ---- combine the 16 waves pairwise, normalise, store ----
-    // thread -> (head, adjacent dim pair)
+    // ---- combine the 16 virtual waves pairwise, normalise, store: thread -> (head, dim pair) ----
     if (c.tid < G * D / 2) {
         const int h = c.tid / (D / 2), d = (c.tid % (D / 2)) * 2;
-        float o0[kWaves], o1[kWaves], l[kWaves];
+        float o0[kVirtualWaves], o1[kVirtualWaves], l[kVirtualWaves];
 #pragma unroll
-        for (int w = 0; w < kWaves; w++) {
+        for (int w = 0; w < kVirtualWaves; w++) {
             o0[w] = sm->wave_o[w][h][d];
             o1[w] = sm->wave_o[w][h][d + 1];
             l[w] = sm->wave_l[w][h];
         }
 #pragma unroll
-        for (int s = 1; s < kWaves; s <<= 1)
+        for (int s = 1; s < kVirtualWaves; s <<= 1)
 #pragma unroll
-            for (int i = 0; i < kWaves; i += 2 * s) {
+            for (int i = 0; i < kVirtualWaves; i += 2 * s) {
                 o0[i] = o0[i] + o0[i + s];
                 o1[i] = o1[i] + o1[i + s];
                 l[i] = l[i] + l[i + s];
@@ -713,7 +930,8 @@ __device__ bool op_attention(const Ctx &c, const int *ins) {
         } else {
             r0 = o0[0] / l[0];
             r1 = o1[0] / l[0];
-            lse = (sm->head_m[h] * 1.44269504088896341f) + mkm::log2f_exact(l[0]);
+            const float m = h == 0 ? hm[0] : h == 1 ? hm[1] : h == 2 ? hm[2] : hm[3];
+            lse = (m * 1.44269504088896341f) + mkm::log2f_exact(l[0]);
         }
         if (skip) {
             st_u32(a.attn_out + (size_t)head * D + d, mkm::pack_bf16(r0, r1));
@@ -724,12 +942,8 @@ __device__ bool op_attention(const Ctx &c, const int *ins) {
             if (d == 0) st_f32(a.attn_lse_intermediates + (size_t)head * a.max_partials + pidx, lse);
         }
     }
-    __syncthreads();
-    if (skip) {
-        if (c.tid == 0) signal_sharded(c, layer, 2, G);
-    } else {
-        if (c.tid < G) add_i32(bar_ptr(c, layer, 1, h0 + c.tid), 1);
-    }
+    wait_stores();
+    wg_barrier();
     return true;
 }
 
@@ -737,33 +951,38 @@ __device__ bool op_attention(const Ctx &c, const int *ins) {
 // opcode 3: log-sum-exp merge of attention partitions  (python_vm.py:349-393;
 // reference device op: demos/low-latency-llama/attention_reduction.cu:18-339)
 // ---------------------------------------------------------------------------------------------
-__device__ bool op_attention_reduction(const Ctx &c, const int *ins) {
+__device__ __forceinline__ bool op_attention_reduction(const Ctx &c, const int *ins) {
     const mk_llama_args &a = c.a;
     Smem *sm = c.sm;
     const int layer = ins[1], hs = ins[2], P = ins[3], terminal = ins[4], n = ins[5];
     const int D = a.head_dim, R = a.attn_reduction_size, MP = a.max_partials;
     bool bad = layer < 0 || layer >= a.num_layers || n < 1 || n > MK_INSTRUCTION_WORDS - 7 || hs < 0 ||
-               hs + R > a.num_attention_heads || R > kGqaMax;
+               hs + R > a.num_attention_heads || R > kGqa;
     if (!bad)
         for (int i = 0; i < n; i++) bad |= ins[6 + i] < 0 || ins[6 + i] >= MP;
     const int out_idx = bad ? 0 : ins[6 + n];
     bad |= !terminal && (out_idx < 0 || out_idx >= MP);
     if (bad) return bail(c, MK_STATUS_BAD_INSTRUCTION);
-    const bool ok = wait_dependency(c, [&]() {
-        const int *p = c.lane < R ? bar_ptr(c, layer, 1, hs + c.lane) : nullptr;
-        return poll_wave0(c, p, false, P);
-    });
-    if (!ok) return false;
 
-    // weights 2^(lse_i - max) once per (head, list entry)
-    if (c.tid < R) {
-        const float *lses = a.attn_lse_intermediates + (size_t)(hs + c.tid) * MP;
-        float m = -INFINITY;
-        for (int i = 0; i < n; i++) m = fmaxf(m, ld_f32(lses + ins[6 + i]));
-        sm->head_m[c.tid] = m;
-        for (int i = 0; i < n; i++) sm->head_w[c.tid][i] = mkm::exp2f_exact(ld_f32(lses + ins[6 + i]) - m);
+    if (c.controller) {
+        const int *p = c.lane < R ? bar_ptr(c, layer, 1, hs + c.lane) : nullptr;
+        const bool ok = poll_counters(c, p, false, P);
+        trace_event(c, kEvDepReady);
+        if (ok && c.lane < R) {
+            // weights 2^(lse_i - max) once per (head, list entry)
+            const float *lses = a.attn_lse_intermediates + (size_t)(hs + c.lane) * MP;
+            float m = -INFINITY;
+            for (int i = 0; i < n; i++) m = fmaxf(m, ld_f32(lses + ins[6 + i]));
+            sm->head_m[c.lane] = m;
+            for (int i = 0; i < n; i++) sm->head_w[c.lane][i] = mkm::exp2f_exact(ld_f32(lses + ins[6 + i]) - m);
+        }
+        if (!barrier_inputs_ready(c, ok)) return false;
+        wg_barrier();  // outputs stored
+        trace_event(c, kEvComputeDone);
+        signal_sharded(c, layer, 2, R);
+        return true;
     }
-    __syncthreads();
+    if (!barrier_inputs_ready(c, true)) return false;
     if (c.tid < R * D / 2) {
         const int h = c.tid / (D / 2), d = (c.tid % (D / 2)) * 2;
         const int head = hs + h;
@@ -788,8 +1007,8 @@ __device__ bool op_attention_reduction(const Ctx &c, const int *ins) {
                 st_f32(a.attn_lse_intermediates + (size_t)head * MP + out_idx, sm->head_m[h] + mkm::log2f_exact(den));
         }
     }
-    __syncthreads();
-    if (c.tid == 0) signal_sharded(c, layer, 2, R);
+    wait_stores();
+    wg_barrier();
     return true;
 }
 
@@ -812,16 +1031,20 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
           (int)threadIdx.x,
           (int)threadIdx.x / 64,
           (int)threadIdx.x % 64,
+          (int)threadIdx.x / 64 == kConsumerWaves,
           (int)blockIdx.x,
           0,
           0,
           (long long)(a.spin_limit_us ? a.spin_limit_us : 2000000u) * 100,
-          a.num_attention_heads + 2 * a.num_kv_heads};
+          a.num_attention_heads + 2 * a.num_kv_heads,
+          nullptr,
+          wall_clock64()};
+    const bool tracing = (a.flags & MK_FLAG_TIMINGS) && a.timings;
     if (c.tid == 0) {
         sm->abort = 0;
         sm->last_flag = 0;
     }
-    __syncthreads();
+    wg_barrier();
 
     const int *queue = a.instructions + (size_t)c.worker * a.num_slots * MK_INSTRUCTION_WORDS;
     for (int slot = 0; slot < a.num_slots; slot++) {
@@ -829,6 +1052,11 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
         const int opcode = ins[0];
         c.slot = slot;
         c.opcode = opcode;
+        if (tracing) {
+            c.trace = a.timings + ((size_t)c.worker * a.num_slots + slot) * MK_TIMING_SLOTS;
+            trace_event(c, kEvStart);
+            if (c.controller && c.lane == 0) c.trace[kEvOpcode] = opcode;
+        }
         bool ok = true;
         switch (opcode) {
         case 0: break;  // NoOp pads the queues (megakernels/scheduler.py:287-289)
@@ -841,17 +1069,19 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
         case 7: ok = op_lm_head<KC_HID>(c, ins); break;
         default: ok = bail(c, MK_STATUS_BAD_OPCODE);  // reference: trap, include/util.cuh:38
         }
+        trace_event(c, kEvEnd);
         if (!ok) break;
     }
 
     // The last workgroup to get here folds the sharded counters into `barriers` and leaves the
     // shards zeroed for the next launch.
-    __syncthreads();  // this workgroup's atomics and stores are complete
+    wait_stores();
+    wg_barrier();
     if (c.tid == 0) {
         const int done = __hip_atomic_fetch_add(&c.status[kDoneSlot], 1, __ATOMIC_RELAXED, AG);
         sm->last_flag = done == (int)gridDim.x - 1;
     }
-    __syncthreads();
+    wg_barrier();
     if (sm->last_flag) {
         const int counters = a.num_layers * kHotRows;
         for (int i = c.tid; i < counters; i += kThreads) {
@@ -935,11 +1165,11 @@ int mk_llama_launch(const mk_llama_args *args, void *hip_stream) {
     }
     const int hid = a.hidden_size, R = a.matvec_reduction_size, D = a.head_dim;
     if (a.num_layers <= 0 || a.num_workers <= 0 || a.num_slots <= 0) return fail(-3, "empty model or schedule");
-    if (a.num_attention_heads != a.num_kv_heads * kGqaMax)
+    if (a.num_attention_heads != a.num_kv_heads * kGqa)
         return fail(-3, "unsupported head grouping: %d query heads for %d KV heads (need %d per KV head)",
-                    a.num_attention_heads, a.num_kv_heads, kGqaMax);
+                    a.num_attention_heads, a.num_kv_heads, kGqa);
     if (a.num_attention_heads * D != hid) return fail(-3, "num_attention_heads * head_dim must equal hidden_size");
-    if (a.attn_reduction_size != kGqaMax) return fail(-3, "attn_reduction_size must be %d", kGqaMax);
+    if (a.attn_reduction_size != kGqa) return fail(-3, "attn_reduction_size must be %d", kGqa);
     if (R <= 0 || hid % R || a.intermediate_size % R) return fail(-3, "sizes are not multiples of the reduction width");
     if (a.vocab_size % 16 || a.intermediate_size % 16) return fail(-3, "vocab and intermediate sizes must be multiples of 16");
     if (a.pos_id < 0 || a.pos_id >= a.kv_max_len || a.pos_id >= a.rope_positions)

@@ -50,6 +50,8 @@ _workspaces: dict[tuple, torch.Tensor] = {}
 
 # barrier waits give up after this many microseconds (0 = library default)
 spin_limit_us = 0
+# set to True to have every launch fill the `timings` tensor (see MK_FLAG_TIMINGS in mk_llama.h)
+record_timings = False
 
 
 def load_library():
@@ -180,7 +182,7 @@ def mk_llama(
     a.workspace = ws.data_ptr()
     a.workspace_bytes = ws.numel() * 4
     a.spin_limit_us = int(spin_limit_us)
-    a.flags = 0
+    a.flags = 1 if (record_timings and timings is not None) else 0
 
     if stream is None:
         stream = torch.cuda.current_stream(barriers.device)
