@@ -52,17 +52,21 @@ constexpr int kShards = 16;         // shards per hot barrier counter
 constexpr int kHotRows = 4;         // barrier rows 2..5 are sharded
 constexpr int kOutRows = 2048;      // rows staged in LDS between matvec and epilogue
 constexpr int kMaxK = 4096;         // longest activation vector handed through LDS
-constexpr int kScoreCap = 6144;     // tokens per attention partition (LDS score buffer)
+constexpr int kScoreCap = 4096;     // tokens per attention partition (LDS score buffer)
+constexpr int kQueueSlots = 192;    // instructions of this worker's queue kept in LDS
 constexpr int kMaxHeadDim = 128;
 constexpr int kGqa = 4;             // query heads per KV head handled by one attention instruction
 constexpr int kStatusInts = 16;
 constexpr int kDoneSlot = 8;        // workspace int: workgroups finished
 
-// Weight rows in flight per consumer wave.  16 VGPRs per 2048-element row; the 9-wave workgroup
-// leaves each lane 168 VGPRs.  8 waves x 4 rows x 4 KB = 128 KB per CU covers the ~4 us a worker
-// spends between two instructions at its ~31 GB/s share of HBM bandwidth.
+// Weight rows in flight per consumer wave (16 VGPRs per 2048-element row; the 9-wave workgroup
+// leaves each lane 168 VGPRs).  8 waves x 3 rows x 4 KB = 96 KB per CU; measured on MI355X, 2, 3, 4
+// and 6 rows stream equally fast, and deeper queues only delay the controller's small loads.
+#ifndef MK_ROWS_IN_FLIGHT
+#define MK_ROWS_IN_FLIGHT 3
+#endif
 template <int KC>
-constexpr int rows_in_flight() { return KC <= 4 ? 4 : 2; }
+constexpr int rows_in_flight() { return KC <= 4 ? MK_ROWS_IN_FLIGHT : 2; }
 
 #define AG __HIP_MEMORY_SCOPE_AGENT
 
@@ -104,6 +108,7 @@ struct Smem {
     float head_w[kGqa][32];         // reduction weights
     float wave_o[kVirtualWaves][kGqa][kMaxHeadDim];
     float scores[kGqa][kScoreCap];
+    int queue[kQueueSlots][MK_INSTRUCTION_WORDS];  // this worker's instructions, fetched once
 };
 static_assert(sizeof(Smem) <= 160 * 1024, "LDS budget");
 static_assert(sizeof(Smem) > 80 * 1024, "must keep a second workgroup off the CU");
@@ -129,8 +134,18 @@ __device__ __forceinline__ uint4 ld_b128(const void *p) {
     uint64_t a = ld_u64(p), b = ld_u64((const char *)p + 8);
     return make_uint4((uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32));
 }
-// immutable data (weights, rope tables, old KV rows): ordinary cached 16-byte load
+// immutable data (rope tables, old KV rows): ordinary cached 16-byte load
 __device__ __forceinline__ uint4 ld_const_b128(const void *p) { return *(const uint4 *)p; }
+// weights: read exactly once per step, so stream them past the caches ("nt")
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 ld_stream_b128(const void *p) {
+#ifdef MK_NO_NT
+    return *(const uint4 *)p;
+#else
+    const u32x4 v = __builtin_nontemporal_load((const u32x4 *)p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+#endif
+}
 
 // All of this wave's global stores and atomics have been performed.  The "memory" clobber keeps
 // the compiler from moving memory operations across it.
@@ -416,7 +431,7 @@ __device__ __forceinline__ void x_from_lds(XVec<KC> &x, const Smem *sm, int lane
 template <int KC>
 __device__ __forceinline__ void load_row(uint4 (&w)[KC], const uint16_t *row, int lane) {
 #pragma unroll
-    for (int j = 0; j < KC; j++) w[j] = ld_const_b128(row + j * 512 + lane * 8);
+    for (int j = 0; j < KC; j++) w[j] = ld_stream_b128(row + j * 512 + lane * 8);
 }
 
 template <int KC>
@@ -440,19 +455,23 @@ __device__ __forceinline__ float dot_row(const uint4 (&w)[KC], const XVec<KC> &x
 //   consumers : request the first rows, barrier (activation vector ready), stream `ntasks` rows
 //               (task t -> wave t % 8, result bf16-rounded into sm->out[t]), barrier (results ready)
 //   controller: `prepare` (wait for the dependency, build the activation vector in LDS; returns
-//               false to abandon), barrier, barrier, `finish` (epilogue + signal)
+//               false to abandon), barrier, `overlap`, barrier, `finish` (epilogue + signal)
 // Both barriers are reached by all nine waves whatever the outcome of `prepare`.
-template <int KC, class RowPtr, class Prepare, class Finish>
+template <int KC, class RowPtr, class Prepare, class Overlap, class Finish>
 __device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need_x, RowPtr row_ptr, Prepare prepare,
-                                             Finish finish) {
+                                             Overlap overlap, Finish finish) {
     constexpr int PF = rows_in_flight<KC>();
     if (c.controller) {
         const bool ok = prepare();
         trace_event(c, kEvInputReady);
         if (!barrier_inputs_ready(c, ok)) return false;
+        overlap();  // runs while the consumers stream rows: fetch what the epilogue will need
         wg_barrier();
         trace_event(c, kEvComputeDone);
         finish();
+#ifndef MK_NO_EPILOGUE_FIRST
+        wg_barrier();
+#endif
         return true;
     }
     const int mine = ntasks > c.wave ? (ntasks - c.wave + kConsumerWaves - 1) / kConsumerWaves : 0;
@@ -475,6 +494,11 @@ __device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need
         }
     }
     wg_barrier();
+#ifndef MK_NO_EPILOGUE_FIRST
+    // hold the next instruction's weight requests back until the controller has sent this
+    // instruction's results and signal: they would otherwise queue behind the bulk loads
+    wg_barrier();
+#endif
     return true;
 }
 
@@ -514,6 +538,7 @@ __device__ __forceinline__ bool op_qkv(const Ctx &c, const int *ins) {
             }
             return true;
         },
+        [&]() {},
         [&]() {
             // epilogue: one lane per adjacent row pair
             const int k_start = H * D, v_start = k_start + KVH * D;
@@ -569,6 +594,11 @@ __device__ __forceinline__ bool op_matvec_add(const Ctx &c, const int *ins, bool
     const int wait_row = is_down ? 4 : 2;
     const int wait_target = is_down ? a.intermediate_size / 16 : a.num_attention_heads;
     uint16_t *resid = a.hidden_states;
+    // The residual rows this instruction updates were last written before its dependency was
+    // satisfied, so the controller can fetch them while the consumers work.
+    constexpr int kPre = 2;
+    uint32_t pre[kPre] = {0, 0};
+    const bool prefetched = nblk * 8 <= kPre * 64;
 
     return matvec_batch<KC>(
         c, nblk * 16, nblk > 0, [&](int t) { return W + (size_t)(start * 16 + t) * in_dim; },
@@ -583,10 +613,19 @@ __device__ __forceinline__ bool op_matvec_add(const Ctx &c, const int *ins, bool
             return true;
         },
         [&]() {
+            if (prefetched) {
+#pragma unroll
+                for (int k = 0; k < kPre; k++) {
+                    const int p = c.lane + k * 64;
+                    if (p < nblk * 8) pre[k] = ld_u32(resid + start * 16 + p * 2);
+                }
+            }
+        },
+        [&]() {
             if (ngroups == 1) {
                 for (int p = c.lane; p < nblk * 8; p += 64) {
                     const int row0 = start * 16 + p * 2;
-                    const uint32_t h = ld_u32(resid + row0);
+                    const uint32_t h = prefetched ? (p < 64 ? pre[0] : pre[1]) : ld_u32(resid + row0);
                     const float lo = mkm::bf16_lo(h) + c.sm->out[p * 2];
                     const float hi = mkm::bf16_hi(h) + c.sm->out[p * 2 + 1];
                     st_u32(resid + row0, mkm::pack_bf16(lo, hi));
@@ -606,7 +645,7 @@ __device__ __forceinline__ bool op_matvec_add(const Ctx &c, const int *ins, bool
                 for (int p = c.lane; p < nblk * 8; p += 64) {
                     if (!c.sm->flags[p >> 3]) continue;
                     const int row0 = start * 16 + p * 2;
-                    const uint32_t h = ld_u32(resid + row0);
+                    const uint32_t h = prefetched ? (p < 64 ? pre[0] : pre[1]) : ld_u32(resid + row0);
                     float lo = mkm::bf16_lo(h), hi = mkm::bf16_hi(h);
                     for (int g = 0; g < ngroups; g++) {
                         const uint64_t v = ld_u64(c.partial + (size_t)g * hid + row0);
@@ -657,6 +696,7 @@ __device__ __forceinline__ bool op_upgate(const Ctx &c, const int *ins) {
             }
             return true;
         },
+        [&]() {},
         [&]() {
             for (int p = c.lane; p < n * 8; p += 64) {
                 const int i = p >> 3, r = (p & 7) * 2;
@@ -701,6 +741,7 @@ __device__ __forceinline__ bool op_lm_head(const Ctx &c, const int *ins) {
                 x_to_lds<KC>(x, c.sm, c.lane);
                 return true;
             },
+            [&]() {},
             [&]() {
                 for (int p = c.lane; p < nblk * 8; p += 64)
                     st_u32(a.logits + b0 * 16 + p * 2, mkm::pack_bf16(c.sm->out[p * 2], c.sm->out[p * 2 + 1]));
@@ -1044,11 +1085,19 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
         sm->abort = 0;
         sm->last_flag = 0;
     }
+    // Instruction fetch (reference: controller warp, include/controller/instruction_fetch.cuh:10-27):
+    // the whole queue of this worker is copied into LDS once, so decoding an instruction never
+    // waits on HBM.  Queues longer than the LDS copy are read in place.
+    const int *queue = a.instructions + (size_t)c.worker * a.num_slots * MK_INSTRUCTION_WORDS;
+    {
+        const int words = min(a.num_slots, kQueueSlots) * MK_INSTRUCTION_WORDS;
+        int *dst = &sm->queue[0][0];
+        for (int i = c.tid; i < words; i += kThreads) dst[i] = queue[i];
+    }
     wg_barrier();
 
-    const int *queue = a.instructions + (size_t)c.worker * a.num_slots * MK_INSTRUCTION_WORDS;
     for (int slot = 0; slot < a.num_slots; slot++) {
-        const int *ins = queue + (size_t)slot * MK_INSTRUCTION_WORDS;
+        const int *ins = slot < kQueueSlots ? sm->queue[slot] : queue + (size_t)slot * MK_INSTRUCTION_WORDS;
         const int opcode = ins[0];
         c.slot = slot;
         c.opcode = opcode;

@@ -16,8 +16,11 @@ from pathlib import Path
 
 import torch
 
+import os
+
 _HERE = Path(__file__).resolve().parent
-LIBRARY = _HERE / "libmk_llama.so"
+# MK_LLAMA_LIB selects another build of the same ABI (used when comparing kernel variants)
+LIBRARY = Path(os.environ.get("MK_LLAMA_LIB", _HERE / "libmk_llama.so"))
 
 _P = ctypes.c_void_p
 _I = ctypes.c_int32
