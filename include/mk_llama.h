@@ -114,6 +114,12 @@ int mk_llama_read_status(void *workspace, void *hip_stream, int32_t out[4]);
  * attention partition (tokens) the kernel accepts. */
 int mk_llama_query(int what);
 
+/* Self test (no counterpart in the reference): counts the binary32 inputs, over all 2^32 bit
+ * patterns except NaNs, for which the kernel's one-instruction bf16 conversion differs from the
+ * portable round-to-nearest-even formula.  Synchronous, allocates 8 bytes of device memory; for
+ * test suites, not for the decode path.  Must report 0. */
+int mk_llama_selftest_bf16(uint64_t *mismatches_out);
+
 const char *mk_llama_last_error(void);
 
 #ifdef __cplusplus

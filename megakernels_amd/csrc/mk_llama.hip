@@ -1149,6 +1149,20 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
     }
 }
 
+// Self test: the one-instruction bf16 conversion against the portable round-to-nearest-even formula
+// for every non-NaN binary32 input.  Each thread walks a strided slice of the 2^32 bit patterns.
+__global__ void bf16_convert_sweep_kernel(unsigned long long *mismatches) {
+    const uint32_t stride = gridDim.x * blockDim.x;
+    unsigned long long bad = 0;
+    uint32_t bits = blockIdx.x * blockDim.x + threadIdx.x;
+    for (uint64_t i = bits; i < (1ull << 32); i += stride) {
+        const float f = mkm::bits_f32((uint32_t)i);
+        if (f != f) continue;
+        bad += mkm::f32_to_bf16(f) != mkm::f32_to_bf16_soft(f);
+    }
+    if (bad) atomicAdd(mismatches, bad);
+}
+
 // ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
@@ -1255,6 +1269,22 @@ int mk_llama_launch(const mk_llama_args *args, void *hip_stream) {
     hipLaunchKernelGGL(fn, dim3(a.num_workers), dim3(kThreads), sizeof(Smem), (hipStream_t)hip_stream, a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(-9, "kernel launch: %s", hipGetErrorString(e));
+    return 0;
+}
+
+int mk_llama_selftest_bf16(uint64_t *mismatches_out) {
+    g_error[0] = 0;
+    if (!mismatches_out) return fail(-1, "null pointer");
+    unsigned long long *dev = nullptr;
+    hipError_t e = hipMalloc(&dev, sizeof *dev);
+    if (e != hipSuccess) return fail(-9, "hipMalloc: %s", hipGetErrorString(e));
+    hipMemset(dev, 0, sizeof *dev);
+    hipLaunchKernelGGL(bf16_convert_sweep_kernel, dim3(4096), dim3(256), 0, 0, dev);
+    unsigned long long host = 0;
+    e = hipMemcpy(&host, dev, sizeof host, hipMemcpyDeviceToHost);
+    hipFree(dev);
+    if (e != hipSuccess) return fail(-9, "self test: %s", hipGetErrorString(e));
+    *mismatches_out = host;
     return 0;
 }
 

@@ -109,3 +109,21 @@ def mismatches(g_ref, g_dev, names=None, kv_rows=None):
         if n:
             report[name] = n
     return report
+
+
+class _Holder:
+    def __init__(self, **kw):
+        self.__dict__.update(kw)
+
+
+def shape_only_model(cfg, max_len=64):
+    """A stand-in model that carries the architecture and zero-element tensors:
+    enough for the scheduler (pure integer logic), far too little to run."""
+    empty = torch.empty(0, dtype=torch.bfloat16)
+    params = _Holder(qkv_proj=empty, o_proj=empty, attn_ln_weight=empty, mlp_ln_weight=empty,
+                     up_proj=empty, gate_proj=empty, down_proj=empty)
+    return _Holder(
+        config=cfg, device=torch.device("cpu"), dtype=torch.bfloat16, stacked_params=params,
+        lm_head=_Holder(input_norm=_Holder(weight=empty), lm_head=_Holder(weight=empty)),
+        stacked_kv_cache=(empty, empty), model=_Holder(rope_cos=empty, rope_sin=empty),
+    )

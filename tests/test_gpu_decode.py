@@ -1,0 +1,179 @@
+"""GPU: multi-step greedy decoding through the reference-shaped generator loop
+(embedding, barrier reset, megakernel, argmax) must produce the checker's token
+ids bit for bit and leave the same KV cache behind; plus the behaviour of the
+launch boundary when things go wrong (every kernel still exits normally)."""
+
+import ctypes
+import sys
+
+import pytest
+import torch
+
+from helpers import (
+    build_schedule, config_1b_slice, config_8b_slice, config_tiny, fill_kv, make_model, mirror_to_gpu, mismatches,
+)
+
+pytestmark = pytest.mark.gpu
+
+
+def _interpreter():
+    from megakernels_amd.demos.latency.mk import LatencyMK_Interpreter
+    return LatencyMK_Interpreter(), sys.modules["mk_llama"]
+
+
+def _decode_case(cfg, workers, prefill, ntok, partitions=1, max_len=256, sched="rr"):
+    from megakernels_amd.generators import MK_Generator
+    from oracle import pyvm
+
+    print(f"decode case hidden={cfg.hidden_size} workers={workers} prefill={prefill} ntok={ntok} "
+          f"partitions={partitions}", flush=True)
+    model = make_model(cfg, max_len=max_len)
+    fill_kv(model, upto=prefill)
+    schedule = build_schedule(model, workers, partitions=partitions, sched=sched)
+    model_gpu, schedule_gpu = mirror_to_gpu(model, schedule)
+    interp, mk_mod = _interpreter()
+
+    tokens_cpu = torch.zeros(1, ntok + 1, dtype=torch.long)
+    tokens_cpu[0, 0] = 5
+    pyvm.OracleGenerator(model, schedule).generate(tokens_cpu, prompt_len=prefill, ntok=ntok)
+
+    tokens_gpu = torch.zeros(1, ntok + 1, dtype=torch.long, device="cuda:0")
+    tokens_gpu[0, 0] = 5
+    MK_Generator(model_gpu, interp, schedule_gpu).generate(tokens_gpu, prompt_len=prefill, ntok=ntok)
+    mk_mod.check_status("cuda:0")
+    assert tokens_gpu.cpu().tolist() == tokens_cpu.tolist()
+    rows = slice(prefill, prefill + ntok)
+    report = mismatches(schedule.globs, schedule_gpu.globs, kv_rows=rows)
+    assert not report, report
+
+
+def test_decode_tiny():
+    _decode_case(config_tiny(), workers=16, prefill=20, ntok=12)
+
+
+def test_decode_tiny_split_kv_crossing_block_boundaries():
+    # positions 30..49 cross the 16-token block boundaries at 32 and 48
+    _decode_case(config_tiny(), workers=16, prefill=30, ntok=20, partitions=3)
+
+
+def test_decode_1b_slice():
+    _decode_case(config_1b_slice(layers=3), workers=256, prefill=100, ntok=8)
+
+
+def test_decode_1b_slice_long_context_split_kv():
+    _decode_case(config_1b_slice(layers=2), workers=256, prefill=2000, ntok=6, partitions=9, max_len=2048 + 64)
+
+
+def test_decode_8b_slice():
+    _decode_case(config_8b_slice(layers=2), workers=256, prefill=50, ntok=4, partitions=2)
+
+
+def test_hardware_bf16_conversion_equals_portable_formula():
+    _, mk_mod = _interpreter()
+    lib = mk_mod.load_library()
+    lib.mk_llama_selftest_bf16.argtypes = [ctypes.POINTER(ctypes.c_uint64)]
+    out = ctypes.c_uint64(123)
+    assert lib.mk_llama_selftest_bf16(ctypes.byref(out)) == 0
+    assert out.value == 0
+
+
+def test_timings_are_recorded_on_request():
+    model = make_model(config_tiny())
+    fill_kv(model, upto=9)
+    schedule = build_schedule(model, 16)
+    schedule.globs.pos_id = 9
+    _, schedule_gpu = mirror_to_gpu(model, schedule)
+    interp, mk_mod = _interpreter()
+    g = schedule_gpu.globs
+    interp.interpret(g)
+    mk_mod.check_status("cuda:0")
+    assert int(g.timings.abs().sum()) == 0          # off by default, like the reference build
+    mk_mod.record_timings = True
+    try:
+        g.barriers.zero_()
+        interp.interpret(g)
+        mk_mod.check_status("cuda:0")
+    finally:
+        mk_mod.record_timings = False
+    t = g.timings.cpu()
+    ins = g.instructions.cpu()
+    real = ins[:, :, 0] != 0
+    assert torch.equal(t[:, :, 5][real], ins[:, :, 0][real])            # opcode echoed
+    assert bool((t[:, :, 4][real] >= t[:, :, 0][real]).all())            # end after start
+    assert bool((t[:, :, 1][real] >= t[:, :, 0][real]).all())            # dependency seen after start
+
+
+def test_unsatisfiable_dependency_times_out_and_reports():
+    """A schedule whose attention never runs: the O projection's wait can never be satisfied.  With
+    a short spin limit the workers give up, record the status and exit; nothing hangs."""
+    model = make_model(config_tiny())
+    fill_kv(model, upto=9)
+    schedule = build_schedule(model, 16)
+    g = schedule.globs
+    g.pos_id = 9
+    g.instructions[g.instructions[:, :, 0] == 2] = 0   # drop every attention instruction
+    _, schedule_gpu = mirror_to_gpu(model, schedule)
+    interp, mk_mod = _interpreter()
+    mk_mod.spin_limit_us = 20000
+    try:
+        interp.interpret(schedule_gpu.globs)
+        code, worker, slot, opcode = mk_mod.read_status("cuda:0")
+    finally:
+        mk_mod.spin_limit_us = 0
+    assert code == 1 and opcode == 4
+    with pytest.raises(RuntimeError, match="timed out"):
+        mk_mod.spin_limit_us = 20000
+        try:
+            schedule_gpu.globs.barriers.zero_()
+            interp.interpret(schedule_gpu.globs)
+            mk_mod.check_status("cuda:0")
+        finally:
+            mk_mod.spin_limit_us = 0
+    # the workspace was cleaned: a valid schedule runs right after
+    test_decode_tiny()
+
+
+def test_unknown_opcode_and_bad_fields_are_reported():
+    model = make_model(config_tiny())
+    schedule = build_schedule(model, 16)
+    g = schedule.globs
+    g.pos_id = 3
+    _, schedule_gpu = mirror_to_gpu(model, schedule)
+    interp, mk_mod = _interpreter()
+    gg = schedule_gpu.globs
+    good = gg.instructions.clone()
+    mk_mod.spin_limit_us = 20000
+    try:
+        gg.instructions[3, 0, 0] = 42
+        interp.interpret(gg)
+        code, worker, slot, opcode = mk_mod.read_status("cuda:0")
+        assert (code, worker, slot, opcode) == (2, 3, 0, 42)
+        gg.instructions.copy_(good)
+        gg.instructions[2, 0, 1] = 99                  # layer index out of range
+        gg.barriers.zero_()
+        interp.interpret(gg)
+        assert mk_mod.read_status("cuda:0")[0] == 4
+    finally:
+        mk_mod.spin_limit_us = 0
+
+
+def test_launch_argument_validation():
+    model = make_model(config_tiny())
+    schedule = build_schedule(model, 16)
+    _, schedule_gpu = mirror_to_gpu(model, schedule)
+    interp, mk_mod = _interpreter()
+    gg = schedule_gpu.globs
+    gg.pos_id = 10_000_000
+    with pytest.raises(RuntimeError, match="pos_id"):
+        interp.interpret(gg)
+    gg.pos_id = 1
+    saved = gg.logits
+    gg.logits = torch.zeros(7, dtype=torch.bfloat16, device="cuda:0")
+    with pytest.raises(RuntimeError, match="logits"):
+        interp.interpret(gg)
+    gg.logits = saved
+    saved = gg.instructions
+    gg.instructions = saved[:, :, :16].contiguous()
+    with pytest.raises(RuntimeError, match="instructions"):
+        interp.interpret(gg)
+    gg.instructions = saved

@@ -1,0 +1,217 @@
+"""Host-side mirror of the reference's Python surface: model container, rotary
+tables, generators, dispatch, and the mk_dir discovery contract."""
+
+import sys
+import types
+
+import pytest
+import torch
+
+from helpers import build_schedule, config_tiny, fill_kv, make_model
+from megakernels_amd import dispatch
+from megakernels_amd.generators import MK_Generator, PyTorchGenerator
+from megakernels_amd.llama import (
+    LlamaConfig, LlamaForCausalLM, interleave_permutation, rope_inverse_frequencies, rope_tables,
+)
+from megakernels_amd.mk import MK_Interpreter, get_mk_func
+from megakernels_amd.model_types import BatchState, ExtraModelConfig
+from megakernels_amd.utils import assert_div, get_sm_count, set_sm_count_override
+
+
+def test_utils():
+    assert assert_div(12, 4) == 3
+    with pytest.raises(AssertionError):
+        assert_div(13, 4)
+    set_sm_count_override(132)
+    assert get_sm_count("cpu") == 132
+    set_sm_count_override(None)
+    assert get_sm_count("cpu") == 256  # MI355X default when no GPU is visible
+    with pytest.raises(ValueError):
+        set_sm_count_override(0)
+
+
+def test_rope_frequencies_match_transformers_llama3_scaling():
+    """The closed-form llama3 scaling against the third-party implementation the reference
+    uses (transformers' rope utilities), for both model families."""
+    try:
+        from transformers import LlamaConfig as HFConfig
+        from transformers.modeling_rope_utils import ROPE_INIT_FUNCTIONS
+    except Exception as exc:  # pragma: no cover
+        pytest.skip(f"transformers rope utilities not importable: {exc}")
+    for cfg in (LlamaConfig.llama_1b(), LlamaConfig.llama_8b()):
+        scaling = dict(cfg.rope_scaling)
+        hf = HFConfig(hidden_size=cfg.hidden_size, num_attention_heads=cfg.num_attention_heads,
+                      num_key_value_heads=cfg.num_key_value_heads, head_dim=cfg.head_dim,
+                      rope_theta=cfg.rope_theta, max_position_embeddings=cfg.max_position_embeddings,
+                      rope_scaling=scaling)
+        try:
+            inv_freq, attention_factor = ROPE_INIT_FUNCTIONS["llama3"](hf, "cpu")
+        except Exception as exc:  # pragma: no cover - API drift between transformers versions
+            pytest.skip(f"transformers llama3 rope init not callable here: {exc}")
+        assert attention_factor == 1.0
+        ours = rope_inverse_frequencies(cfg)
+        assert torch.allclose(ours, inv_freq, rtol=1e-6, atol=0)
+
+
+def test_rope_tables_layout():
+    cfg = config_tiny()
+    cos, sin = rope_tables(cfg, 32)
+    D = cfg.head_dim
+    assert cos.shape == (32, D) and cos.dtype == torch.float32
+    assert torch.equal(cos[:, : D // 2], cos[:, D // 2:])            # half-split layout
+    assert torch.equal(cos[0], torch.ones(D)) and torch.equal(sin[0], torch.zeros(D))
+    perm = interleave_permutation(D)
+    assert perm[:4].tolist() == [0, D // 2, 1, D // 2 + 1]
+    il = cos[:, perm]
+    assert torch.equal(il[:, 0::2], il[:, 1::2])                      # pairs share a frequency
+    model = make_model(cfg)
+    assert torch.equal(model.model.rope_cos[:32], il)
+
+
+def test_from_random_is_reproducible_and_tied():
+    cfg = config_tiny()
+    a, b = make_model(cfg, seed=5), make_model(cfg, seed=5)
+    for name in vars(a.stacked_params):
+        assert torch.equal(getattr(a.stacked_params, name), getattr(b.stacked_params, name))
+    assert a.lm_head.lm_head.weight is a.model.embed_tokens.weight      # tied, as Llama-3.2-1B
+    c = make_model(cfg, seed=6)
+    assert not torch.equal(a.stacked_params.up_proj, c.stacked_params.up_proj)
+    p = a.stacked_params
+    L, H, KVH, D = cfg.num_hidden_layers, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    assert p.qkv_proj.shape == (L, (H + 2 * KVH) * D, cfg.hidden_size)
+    assert p.down_proj.shape == (L, cfg.hidden_size, cfg.intermediate_size)
+    assert a.stacked_kv_cache[0].shape == (L, 1, 256, KVH, D)
+    assert abs(float(p.up_proj.float().std()) - 0.02) < 2e-3
+    untied = LlamaForCausalLM.from_random(
+        LlamaConfig(hidden_size=512, intermediate_size=1024, num_hidden_layers=1, num_attention_heads=8,
+                    num_key_value_heads=2, vocab_size=1024, tie_word_embeddings=False, max_position_embeddings=64),
+        ExtraModelConfig(interleave_rope=True, max_len_override=16))
+    assert untied.lm_head.lm_head.weight is not untied.model.embed_tokens.weight
+
+
+def test_forward_prefill_equals_token_by_token_decode():
+    cfg = config_tiny()
+    model = make_model(cfg, max_len=32, seed=1)
+    ids = torch.randint(0, cfg.vocab_size, (1, 9), generator=torch.Generator().manual_seed(0))
+    full = model(BatchState(input_ids=ids, position_ids=torch.arange(9)))
+    kv_full = [c.clone() for c in model.stacked_kv_cache]
+    model.setup_caches()
+    outs = []
+    for t in range(9):
+        step = model(BatchState(input_ids=ids[:, t:t + 1], position_ids=torch.tensor([t]), seq_len=t + 1))
+        outs.append(step.hidden_states[:, 0])
+    stepwise = torch.stack(outs, dim=1)
+    assert (stepwise.float() - full.hidden_states.float()).abs().max() <= 2e-2 * full.hidden_states.float().abs().max()
+    for a, b in zip(kv_full, model.stacked_kv_cache):
+        assert (a[:, :, :9].float() - b[:, :, :9].float()).abs().max() <= 2e-2 * a.float().abs().max()
+
+
+def test_interleaved_and_half_split_models_agree():
+    cfg = config_tiny()
+    il = LlamaForCausalLM.from_random(cfg, ExtraModelConfig(interleave_rope=True, max_len_override=16), seed=2)
+    hs = LlamaForCausalLM.from_random(cfg, ExtraModelConfig(interleave_rope=False, max_len_override=16), seed=2)
+    ids = torch.randint(0, cfg.vocab_size, (1, 6), generator=torch.Generator().manual_seed(3))
+    a = il(BatchState(input_ids=ids, position_ids=torch.arange(6)))
+    b = hs(BatchState(input_ids=ids, position_ids=torch.arange(6)))
+    assert (a.hidden_states.float() - b.hidden_states.float()).abs().max() <= 2e-2 * b.hidden_states.float().abs().max()
+
+
+class _RecordingInterpreter:
+    def __init__(self):
+        self.calls = []
+
+    def interpret(self, globs):
+        self.calls.append((int(globs.pos_id), globs.barriers.clone(), globs.hidden_states.clone()))
+        globs.logits.zero_()
+        globs.logits[7] = 1.0
+        globs.logits[9] = 1.0  # tie: argmax must pick index 7
+
+
+def test_mk_generator_loop_semantics():
+    """generators.py:121-163: embedding row into hidden_states, barrier fill, pos_id =
+    prompt_len + already + i - 1, argmax with first-maximum tie break, token written at src + 1."""
+    cfg = config_tiny()
+    model = make_model(cfg)
+    sched = build_schedule(model, 16)
+    interp = _RecordingInterpreter()
+    gen = MK_Generator(model, interp, sched, barrier_fill_val=3)
+    tokens = torch.zeros(1, 5, dtype=torch.long)
+    tokens[0, 0] = 11
+    gen.generate(tokens, prompt_len=20, ntok=4, ntok_already_generated=1)
+    assert tokens[0].tolist() == [11, 7, 7, 7, 7]
+    assert [c[0] for c in interp.calls] == [20, 21, 22, 23]
+    assert all(bool((c[1] == 3).all()) for c in interp.calls)
+    assert torch.equal(interp.calls[0][2], model.model.embed_tokens.weight[11])
+    assert torch.equal(interp.calls[1][2], model.model.embed_tokens.weight[7])
+    skipping = MK_Generator(model, interp, sched, skip_mk=True)
+    n = len(interp.calls)
+    skipping.run(tokens[:, :1], pos_id=3)
+    assert len(interp.calls) == n
+    gen.replace_with_noops()
+    assert int(sched.globs.instructions.abs().sum()) == 0
+
+
+def test_generate_with_eos_chunks():
+    cfg = config_tiny()
+    model = make_model(cfg)
+    sched = build_schedule(model, 16)
+    gen = MK_Generator(model, _RecordingInterpreter(), sched)
+    tokens = torch.zeros(1, 40, dtype=torch.long)
+    pos, generated = gen.generate_with_eos(tokens, prompt_len=4, ntok=40, eos_token_check_interval=16, eos_token_ids=[7])
+    assert (pos, generated) == (1, 16)
+    pos, generated = gen.generate_with_eos(tokens, prompt_len=4, ntok=40, eos_token_check_interval=16, eos_token_ids=[99])
+    assert (pos, generated) == (40, 39)
+
+
+def test_pytorch_generator_matches_manual_decode():
+    cfg = config_tiny()
+    model = make_model(cfg, max_len=32, seed=1)
+    ids = torch.randint(0, cfg.vocab_size, (1, 5), generator=torch.Generator().manual_seed(0))
+    out = model(BatchState(input_ids=ids, position_ids=torch.arange(5)))
+    tokens = torch.zeros(1, 4, dtype=torch.long)
+    tokens[0, 0] = out.output_ids[0, -1]
+    PyTorchGenerator(model).generate(tokens, prompt_len=5, ntok=3)
+    assert tokens.min() >= 0 and tokens.max() < cfg.vocab_size and int(tokens[0, 1:].abs().sum()) > 0
+
+
+def test_dispatch_and_mk_dir_contract(tmp_path):
+    assert type(dispatch.make_schedule_builder("latency")).__name__ == "LatencyScheduleBuilder"
+    with pytest.raises(ValueError):
+        dispatch.make_schedule_builder("throughput")
+    with pytest.raises(NotImplementedError):
+        dispatch.make_pyvm_interpreter("latency")
+    # mk_dir is put on sys.path and must hold a module `mk_llama` with a callable `mk_llama`
+    saved = sys.modules.pop("mk_llama", None)
+    saved_path = list(sys.path)
+    # the directory is appended (as the reference does), so an earlier entry would win
+    sys.path[:] = [p for p in sys.path if not p.rstrip("/").endswith("csrc")]
+    try:
+        (tmp_path / "mk_llama.py").write_text("def mk_llama(*a, **k):\n    return 'called'\n")
+        func = get_mk_func(tmp_path)
+        assert func() == "called"
+        with pytest.raises(NotImplementedError):
+            MK_Interpreter(tmp_path).interpret(None)
+    finally:
+        sys.modules.pop("mk_llama", None)
+        if saved is not None:
+            sys.modules["mk_llama"] = saved
+        sys.path[:] = saved_path
+
+
+def test_shim_refuses_cpu_tensors_and_missing_library(monkeypatch):
+    sys.modules.pop("mk_llama", None)
+    from megakernels_amd.mk import DEFAULT_MK_DIR
+    func = get_mk_func(DEFAULT_MK_DIR)
+    model = make_model(config_tiny())
+    sched = build_schedule(model, 16)
+    from megakernels_amd.demos.latency.mk import LatencyMK_Interpreter
+    interp = LatencyMK_Interpreter(DEFAULT_MK_DIR)
+    with pytest.raises(RuntimeError):
+        # no fallback: CPU tensors are refused before anything is launched
+        monkeypatch.setattr(torch.cuda, "current_stream", lambda *a, **k: types.SimpleNamespace(cuda_stream=0))
+        interp.interpret(sched.globs)
+    mod = sys.modules["mk_llama"]
+    monkeypatch.setattr(mod, "_lib", None)
+    monkeypatch.setattr(mod, "LIBRARY", mod.LIBRARY.with_name("missing.so"))
+    with pytest.raises(RuntimeError, match="missing"):
+        mod.load_library()

@@ -1,0 +1,211 @@
+"""Instruction encoding and scheduling: pure integer logic, pinned against
+(a) the reference's own scheduler output for Llama-3.2-1B on 132 and 148
+workers (tests/golden/reference_schedules.json, written by
+tests/golden/make_schedule_fixtures.py), (b) closed forms and coverage
+invariants, and (c) the word layouts the reference's device parsers read."""
+
+import json
+from collections import Counter
+from pathlib import Path
+
+import pytest
+import torch
+
+from helpers import shape_only_model
+from megakernels_amd.demos.latency.instructions import (
+    AttentionReduction, DownProjResidual, LayerNorm_QKV_MatVecRopeAppend, LayerNormDoubleMatVecSiLU,
+    O_ProjResidual, PartialAttention, RMS_LM_Head,
+)
+from megakernels_amd.demos.latency.scheduler import (
+    LatencyScheduleBuilder, MAX_ATTENTION_PARTITIONS, pick_num_attention_partitions,
+)
+from megakernels_amd.instructions import Instruction, NoOp
+from megakernels_amd.llama import LlamaConfig
+from megakernels_amd.scheduler import (
+    assign_to_sms, collect_into_waves, serialize_and_pad, tensorize_instructions,
+)
+from megakernels_amd.utils import set_sm_count_override
+
+GOLDEN = json.loads((Path(__file__).parent / "golden" / "reference_schedules.json").read_text())
+
+
+def build(cfg, workers, **kw):
+    set_sm_count_override(workers)
+    sched = LatencyScheduleBuilder.build(shape_only_model(cfg), **kw)
+    sched.globs.pos_id = 40
+    return sched
+
+
+def cfg_1b(layers=2):
+    return LlamaConfig(num_hidden_layers=layers)
+
+
+# ---- (c) word layouts, as the reference's device code parses them -----------------------------
+
+
+def test_word_layouts():
+    # rms_matvec_rope_append.cu:38-41: [op, layer, start, end]
+    assert LayerNorm_QKV_MatVecRopeAppend(3, 10, 12).serialize() == [1, 3, 10, 12]
+    # attention_partial.cu:46-49: [op, layer, kv_head, num_partials, partial_idx]
+    assert PartialAttention(2, 5, 7, 6).serialize() == [2, 2, 5, 7, 6]
+    # attention_reduction.cu:34-45: [op, layer, head_start, num_partials, is_terminal, n, list..., out]
+    assert AttentionReduction(1, 8, 3, True, [0, 1, 2], None).serialize() == [3, 1, 8, 3, 1, 3, 0, 1, 2, 0]
+    assert AttentionReduction(1, 8, 3, False, [2, 1], 5).serialize() == [3, 1, 8, 3, 0, 2, 2, 1, 5]
+    # matvec_adds.cu:26-34: [op, layer, start, end, reduction_block]
+    assert O_ProjResidual(4, 7, 8, 0).serialize() == [4, 4, 7, 8, 0]
+    assert DownProjResidual(4, 6, 8, 3).serialize() == [6, 4, 6, 8, 3]
+    # upgate.cu:24-26: [op, layer, n, blocks...]
+    assert LayerNormDoubleMatVecSiLU(9, [3, 135, 267]).serialize() == [5, 9, 3, 3, 135, 267]
+    # rms_lm_head.cu:20-22: [op, start, end]
+    assert RMS_LM_Head(100, 161).serialize() == [7, 100, 161]
+    assert NoOp().serialize() == [0]
+    assert serialize_and_pad(NoOp()) == [0] * 32
+    assert len(serialize_and_pad(RMS_LM_Head(1, 2))) == 32
+
+
+def test_words_round_trip():
+    sched = build(cfg_1b(), 132, num_attention_partitions=5)
+    for ins in sched.get_linear_instructions():
+        words = serialize_and_pad(ins)
+        assert Instruction.from_words(words).serialize() == ins.serialize()
+
+
+def test_too_long_instruction_is_rejected():
+    with pytest.raises(AssertionError):
+        serialize_and_pad(LayerNormDoubleMatVecSiLU(0, list(range(30))))
+
+
+# ---- (a) the reference's own output ----------------------------------------------------------------
+
+
+@pytest.mark.parametrize("workers", [132, 148])
+def test_linear_schedule_matches_reference(workers):
+    sched = build(cfg_1b(), workers)
+    ours = [ins.serialize() for ins in sched.get_linear_instructions()]
+    assert ours == GOLDEN[str(workers)]["linear"]
+
+
+@pytest.mark.parametrize("workers", [132, 148])
+@pytest.mark.parametrize("mode", ["rr", "zz", "wave", "dag"])
+def test_assignment_matches_reference(workers, mode):
+    sched = build(cfg_1b(), workers)
+    queues = assign_to_sms(mode, schedule=sched)
+    ours = [[ins.serialize() for ins in q] for q in queues]
+    assert ours == GOLDEN[str(workers)]["queues"][mode]
+
+
+# ---- (b) closed forms and invariants -------------------------------------------------------------
+
+
+@pytest.mark.parametrize("workers", [132, 148, 256])
+def test_instruction_count_closed_form(workers):
+    layers = 3
+    sched = build(cfg_1b(layers), workers)
+    assert len(sched.dag_nodes) == layers * (3 * workers + 136) + workers
+
+
+@pytest.mark.parametrize("cfg,workers", [(cfg_1b(), 132), (cfg_1b(), 256), (LlamaConfig.llama_8b(), 256)])
+def test_every_block_is_covered_exactly_once(cfg, workers):
+    cfg.num_hidden_layers = 2
+    sched = build(cfg, workers)
+    g = sched.globs
+    H, KVH, D = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+    for layer in range(cfg.num_hidden_layers):
+        ins_l = [i for i in sched.get_linear_instructions() if getattr(i, "layer_idx", None) == layer]
+        qkv = Counter(b for i in ins_l if i.opcode() == 1 for b in i.block_indices())
+        assert qkv == Counter(range((H + 2 * KVH) * D // 16))
+        attn = Counter((i.kv_head_idx, i.partial_idx) for i in ins_l if i.opcode() == 2)
+        assert attn == Counter((k, 0) for k in range(KVH))
+        oproj = Counter((i.reduction_block_idx, b) for i in ins_l if i.opcode() == 4
+                        for b in range(i.start_block_idx, i.end_block_idx))
+        assert oproj == Counter((grp, b) for grp in range(g.o_proj_col_groups()) for b in range(cfg.hidden_size // 16))
+        upgate = Counter(b for i in ins_l if i.opcode() == 5 for b in i.block_idxs)
+        assert upgate == Counter(range(cfg.intermediate_size // 16))
+        down = [(i.reduction_block_idx, b) for i in ins_l if i.opcode() == 6
+                for b in range(i.start_block_idx, i.end_block_idx)]
+        # group-major order: the order in which the bf16 partial sums are applied
+        assert down == [(grp, b) for grp in range(g.down_proj_col_groups()) for b in range(cfg.hidden_size // 16)]
+    lm = Counter(b for i in sched.get_linear_instructions() if i.opcode() == 7
+                 for b in range(i.start_output_block_idx, i.end_output_block_idx))
+    assert lm == Counter(range(cfg.vocab_size // 16))
+
+
+def test_barrier_targets_reproduce_the_reference_constants():
+    g = build(cfg_1b(), 132).globs
+    # python_vm.py:110,132,176,255,283-290
+    assert (g.down_proj_total_jobs(), g.o_proj_total_jobs(), g.up_gate_total_blocks(), g.qkv_blocks_per_head()) == (512, 128, 512, 4)
+    g8 = build(LlamaConfig.llama_8b(), 256).globs
+    assert (g8.o_proj_col_groups(), g8.down_proj_col_groups()) == (2, 7)
+    assert g8.down_proj_total_jobs() == 7 * 256 and g8.o_proj_total_jobs() == 512 and g8.qkv_blocks_per_head() == 8
+
+
+def test_qkv_ranges_use_round_half_even():
+    # 192 blocks over 256 workers: b = 0.75; round(0.75 * 2) = round(1.5) = 2, round(0.75 * 6) = round(4.5) = 4
+    sched = build(cfg_1b(1), 256)
+    qkv = [i for i in sched.get_linear_instructions() if i.opcode() == 1]
+    assert len(qkv) == 256
+    assert [(i.start_output_block_idx, i.end_output_block_idx) for i in qkv[:7]] == [
+        (0, 1), (1, 2), (2, 2), (2, 3), (3, 4), (4, 4), (4, 5)]
+    assert sum(1 for i in qkv if i.start_output_block_idx == i.end_output_block_idx) == 64
+
+
+def test_round_robin_queue_property_and_padding():
+    sched = build(cfg_1b(), 132)
+    linear = sched.get_linear_instructions()
+    queues = assign_to_sms("rr", schedule=sched)
+    for w, q in enumerate(queues):
+        assert [i.serialize() for i in q] == [i.serialize() for i in linear[w::132]]
+    tensorize_instructions(sched.globs, queues)
+    ins = sched.globs.instructions
+    longest = -(-len(linear) // 132)
+    assert tuple(ins.shape) == (132, longest, 32) and ins.dtype == torch.int32
+    assert tuple(sched.globs.timings.shape) == (132, longest, 128)
+    short = len(linear) % 132
+    assert bool((ins[short:, -1] == 0).all()) and bool((ins[:short, -1, 0] != 0).all())
+
+
+@pytest.mark.parametrize("mode", ["zz", "wave", "dag"])
+def test_other_policies_are_permutations(mode):
+    sched = build(cfg_1b(), 256)
+    queues = assign_to_sms(mode, schedule=sched)
+    got = Counter(tuple(i.serialize()) for q in queues for i in q)
+    want = Counter(tuple(i.serialize()) for i in sched.get_linear_instructions())
+    assert got == want
+    with pytest.raises(ValueError):
+        assign_to_sms("nope", schedule=sched)
+
+
+def test_collect_into_waves():
+    sched = build(cfg_1b(1), 132)
+    waves = collect_into_waves(sched.get_linear_instructions())
+    assert [w[0].opcode() for w in waves] == [1, 2, 4, 5, 6, 7]
+
+
+def test_stop_after_op_and_layer_limit():
+    sched = build(cfg_1b(4), 132, stop_after_op="oproj", layer_limit=1)
+    ops = {i.opcode() for i in sched.get_linear_instructions()}
+    assert ops == {1, 2, 4}
+    sched = build(cfg_1b(4), 132, layer_limit=2)
+    assert 7 not in {i.opcode() for i in sched.get_linear_instructions()}
+
+
+def test_split_kv_schedule():
+    P = 6
+    sched = build(cfg_1b(1), 256, num_attention_partitions=P)
+    g = sched.globs
+    assert not g.skip_attn_reduction
+    ins = sched.get_linear_instructions()
+    partials = [i for i in ins if i.opcode() == 2]
+    assert [(i.kv_head_idx, i.num_partials, i.partial_idx) for i in partials] == [(k, P, p) for k in range(8) for p in range(P)]
+    reds = [i for i in ins if i.opcode() == 3]
+    assert [i.head_start_idx for i in reds] == list(range(0, 32, 4))
+    assert all(i.is_terminal and i.reduction_list == list(range(P)) and i.num_partials == P for i in reds)
+    # order: partials, then reductions, then O projection
+    kinds = [i.opcode() for i in ins]
+    assert kinds.index(3) > max(j for j, k in enumerate(kinds) if k == 2)
+    assert kinds.index(4) > max(j for j, k in enumerate(kinds) if k == 3)
+    with pytest.raises(AssertionError):
+        build(cfg_1b(1), 256, num_attention_partitions=MAX_ATTENTION_PARTITIONS + 1)
+    assert pick_num_attention_partitions(4096, 64) == 17
+    assert pick_num_attention_partitions(32, 128) == 1
+    assert pick_num_attention_partitions(16384, 64) == 24
