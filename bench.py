@@ -59,6 +59,10 @@ def main():
     ap.add_argument("--cpu-steps", type=int, default=32, help="decode steps timed on the CPU checker (0 = skip)")
     ap.add_argument("--sched", default="rr")
     ap.add_argument("--partitions", type=int, default=0, help="attention partitions (0 = one per 256 positions, max 24)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="after the timed region also run a plain 1 GiB device copy three times, so that a "
+                         "rocprofv3 --pmc run of this command holds a kernel of known traffic to scale "
+                         "FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -159,6 +163,14 @@ def main():
 
     tokens_gpu = output_tokens[0].cpu().tolist()
 
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=device).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)   # elementwise copy kernel: reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
+
     # ---- CPU baseline: the checker on the same decode steps (bounded sample) --
     cpu_baseline = None
     parity = None
@@ -188,6 +200,13 @@ def main():
         agree = sum(int(a == b) for a, b in zip(expect, got))
         parity = {"tokens_compared": n_cpu + 1, "tokens_equal": agree, "bit_exact": agree == n_cpu + 1}
 
+    # HBM bytes per launch measured with rocprofv3 --pmc for this workload (committed summary)
+    traffic = None
+    traffic_file = ROOT / "profiles" / f"mk_llama_kernel_{args.workload}_traffic.json"
+    if traffic_file.exists():
+        measured = json.loads(traffic_file.read_text())
+        traffic = measured["fetch_bytes_per_launch"] + measured["write_bytes_per_launch"]
+
     result = {
         "metric": "batch-1 decode tokens/s (Llama-3.2-1B arch)",
         "value": round(args.steps / elapsed, 2),
@@ -216,7 +235,7 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved_gbps / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            "traffic": traffic,
             "kernel": "mk_llama_kernel<4,4,64>",
             "kernel_us": round(kernel_ms_mean * 1e3, 2),
             "algorithmic_bytes_per_launch": int(bytes_per_step),

@@ -1,0 +1,102 @@
+"""Manual bisection harness, counterpart of the reference's ``scripts/diff_test.py``: run the CPU
+checker and the HIP megakernel on the same random hidden state / KV cache (valid positions N(0,1),
+positions beyond the sequence N(0,100) as poison) and print, per buffer, the largest absolute
+difference, the mean relative difference and the number of differing elements.  Needs a GPU.
+
+    python tests/diff_test.py model=1b layer_limit=1 stop_after_op=oproj prompt_len=10 ntok=10
+    python tests/diff_test.py model=tiny .full num_attention_partitions=3
+
+It lives with the tests because it drives the checker, which the product never imports.
+"""
+
+from __future__ import annotations
+
+import sys
+from dataclasses import dataclass, fields
+from pathlib import Path
+
+import torch
+
+sys.path.insert(0, str(Path(__file__).resolve().parent.parent))
+sys.path.insert(0, str(Path(__file__).resolve().parent))
+
+from helpers import build_schedule, config_8b_slice, config_tiny, fill_kv, make_model, mirror_to_gpu, mismatches  # noqa: E402
+from megakernels_amd.llama import LlamaConfig  # noqa: E402
+
+
+@dataclass
+class ScriptConfig:
+    model: str = "1b"
+    prompt_len: int = 10
+    ntok: int = 10
+    stop_after_op: str | None = None
+    layer_limit: int | None = 1
+    sched: str = "rr"
+    workers: int = 256
+    num_attention_partitions: int = 1
+    barrier_init_val: int = 0
+    noops: bool = False
+
+    def full(self):
+        self.layer_limit = None
+
+
+def parse(argv):
+    cfg = ScriptConfig()
+    for arg in argv:
+        if arg.startswith("."):
+            getattr(cfg, arg[1:])()
+            continue
+        key, _, value = arg.partition("=")
+        current = getattr(cfg, key)
+        if value in ("None", "none"):
+            setattr(cfg, key, None)
+        elif isinstance(current, bool):
+            setattr(cfg, key, value.lower() in ("1", "true"))
+        elif isinstance(current, int) or key in ("layer_limit",):
+            setattr(cfg, key, int(value))
+        else:
+            setattr(cfg, key, value)
+    return cfg
+
+
+def main(config: ScriptConfig):
+    from megakernels_amd.demos.latency.mk import LatencyMK_Interpreter
+    from oracle import pyvm
+
+    arch = {"1b": LlamaConfig.llama_1b(), "8b": LlamaConfig.llama_8b(), "tiny": config_tiny(),
+            "8b_slice": config_8b_slice()}[config.model]
+    if config.layer_limit is not None and config.model in ("1b", "8b"):
+        # building all layers' weights to run one is wasteful: keep two
+        arch.num_hidden_layers = max(2, config.layer_limit)
+    if config.model == "tiny":
+        config.workers = 16
+    seq_len = config.prompt_len + config.ntok
+    model = make_model(arch, max_len=max(256, seq_len + 16))
+    fill_kv(model, upto=seq_len)
+    schedule = build_schedule(model, config.workers, partitions=config.num_attention_partitions,
+                              sched=config.sched, stop_after_op=config.stop_after_op, layer_limit=config.layer_limit)
+    g = schedule.globs
+    g.hidden_states.normal_()
+    g.pos_id = seq_len - 1
+    g.barriers.fill_(config.barrier_init_val)
+    if config.noops:
+        g.instructions.zero_()
+    queue_lengths = [int((q[:, 0] != 0).sum()) for q in g.instructions]
+    print(f"worker queue lengths: min={min(queue_lengths)}, max={max(queue_lengths)}, "
+          f"mean={sum(queue_lengths) / len(queue_lengths):.2f}")
+    _, schedule_gpu = mirror_to_gpu(model, schedule)
+    instructions = [] if config.noops else schedule.get_linear_instructions()
+    pyvm.interpret(g, instructions, check_barriers=config.barrier_init_val == 0)
+    interp = LatencyMK_Interpreter()
+    interp.interpret(schedule_gpu.globs)
+    sys.modules["mk_llama"].check_status("cuda:0")
+    print("done! diffing tensors:")
+    g.diff(schedule_gpu.globs.__class__(**{f.name: (getattr(schedule_gpu.globs, f.name).cpu()
+           if isinstance(getattr(schedule_gpu.globs, f.name), torch.Tensor) else getattr(schedule_gpu.globs, f.name))
+           for f in fields(schedule_gpu.globs)}))
+    print("elements that differ bit for bit:", mismatches(g, schedule_gpu.globs) or "none")
+
+
+if __name__ == "__main__":
+    main(parse(sys.argv[1:]))
