@@ -53,7 +53,7 @@ constexpr int kHotRows = 4;         // barrier rows 2..5 are sharded
 constexpr int kOutRows = 2048;      // rows staged in LDS between matvec and epilogue
 constexpr int kMaxK = 4096;         // longest activation vector handed through LDS
 constexpr int kScoreCap = 4096;     // tokens per attention partition (LDS score buffer)
-constexpr int kQueueSlots = 192;    // instructions of this worker's queue kept in LDS
+constexpr int kQueueSlots = 256;    // longest instruction queue per worker (kept in LDS)
 constexpr int kMaxHeadDim = 128;
 constexpr int kGqa = 4;             // query heads per KV head handled by one attention instruction
 constexpr int kStatusInts = 16;
@@ -98,7 +98,8 @@ __host__ __device__ inline WsLayout ws_layout(int L, int hid, int inter, int R) 
 struct Smem {
     int abort;                      // set once, never cleared during a launch
     int last_flag;
-    int pad[2];
+    long long t_launch;             // wall clock when the workgroup started
+    mk_llama_args args;             // the launch arguments, read from here by every instruction
     int flags[kOutRows / 16];       // per-block "I was the last arriver" (matvec-add)
     float x[kMaxK];                 // activation vector, lane layout [chunk][lane][8]
     float out[kOutRows];            // matvec row results awaiting the epilogue
@@ -116,33 +117,49 @@ static_assert(sizeof(Smem) > 80 * 1024, "must keep a second workgroup off the CU
 // ---------------------------------------------------------------------------------------------
 // agent-coherent memory access (bypass the non-coherent per-XCD L2 contents)
 // ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ int ld_i32(const int *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, AG); }
+// Device pointers reach the instruction handlers through LDS, so the compiler cannot tell their
+// address space; every access casts to the global address space explicitly.  A generic (flat_*)
+// access would count on lgkmcnt as well as vmcnt and couple LDS waits to outstanding weight loads.
+#define MK_GLOBAL __attribute__((address_space(1)))
+template <class T>
+__device__ __forceinline__ MK_GLOBAL T *as_global(T *p) { return (MK_GLOBAL T *)p; }
+
+__device__ __forceinline__ int ld_i32(const int *p) { return __hip_atomic_load(as_global(p), __ATOMIC_RELAXED, AG); }
 __device__ __forceinline__ uint32_t ld_u32(const void *p) {
-    return __hip_atomic_load((const uint32_t *)p, __ATOMIC_RELAXED, AG);
+    return __hip_atomic_load(as_global((const uint32_t *)p), __ATOMIC_RELAXED, AG);
 }
 __device__ __forceinline__ uint64_t ld_u64(const void *p) {
-    return __hip_atomic_load((const uint64_t *)p, __ATOMIC_RELAXED, AG);
+    return __hip_atomic_load(as_global((const uint64_t *)p), __ATOMIC_RELAXED, AG);
 }
 __device__ __forceinline__ float ld_f32(const float *p) { return mkm::bits_f32(ld_u32(p)); }
 __device__ __forceinline__ void st_u32(void *p, uint32_t v) {
-    __hip_atomic_store((uint32_t *)p, v, __ATOMIC_RELAXED, AG);
+    __hip_atomic_store(as_global((uint32_t *)p), v, __ATOMIC_RELAXED, AG);
 }
 __device__ __forceinline__ void st_f32(float *p, float v) { st_u32(p, mkm::f32_bits(v)); }
-__device__ __forceinline__ void st_i32(int *p, int v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, AG); }
-__device__ __forceinline__ void add_i32(int *p, int v) { __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, AG); }
+__device__ __forceinline__ void st_i32(int *p, int v) { __hip_atomic_store(as_global(p), v, __ATOMIC_RELAXED, AG); }
+__device__ __forceinline__ void add_i32(int *p, int v) { __hip_atomic_fetch_add(as_global(p), v, __ATOMIC_RELAXED, AG); }
+__device__ __forceinline__ int add_ret_i32(int *p, int v) {
+    return __hip_atomic_fetch_add(as_global(p), v, __ATOMIC_RELAXED, AG);
+}
 __device__ __forceinline__ uint4 ld_b128(const void *p) {
     uint64_t a = ld_u64(p), b = ld_u64((const char *)p + 8);
     return make_uint4((uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32));
 }
-// immutable data (rope tables, old KV rows): ordinary cached 16-byte load
-__device__ __forceinline__ uint4 ld_const_b128(const void *p) { return *(const uint4 *)p; }
-// weights: read exactly once per step, so stream them past the caches ("nt")
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+// immutable data (rope tables, old KV rows): ordinary cached 16-byte load
+__device__ __forceinline__ uint4 ld_const_b128(const void *p) {
+    const u32x4 v = *as_global((const u32x4 *)p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ float ld_const_f32(const float *p) { return *as_global(p); }
+// plain store of a word nobody else reads during the launch (timing trace)
+__device__ __forceinline__ void st_plain_i32(int *p, int v) { *as_global(p) = v; }
+// weights: read exactly once per step, so stream them past the caches ("nt")
 __device__ __forceinline__ uint4 ld_stream_b128(const void *p) {
 #ifdef MK_NO_NT
-    return *(const uint4 *)p;
+    return ld_const_b128(p);
 #else
-    const u32x4 v = __builtin_nontemporal_load((const u32x4 *)p);
+    const u32x4 v = __builtin_nontemporal_load(as_global((const u32x4 *)p));
     return make_uint4(v.x, v.y, v.z, v.w);
 #endif
 }
@@ -277,21 +294,72 @@ __device__ __forceinline__ float group_tree_sum(float v) {
 // ---------------------------------------------------------------------------------------------
 // per-workgroup context
 // ---------------------------------------------------------------------------------------------
+// LDS is always addressed through address-space-qualified pointers (ds_* instructions, counted by
+// lgkmcnt).  A generic pointer would turn every access into a flat_* instruction, which also counts
+// on vmcnt and would make LDS reads wait, in order, behind the consumers' outstanding weight loads.
+// The launch arguments and the instruction words live in LDS for the same reason: the instruction
+// handlers are separate functions (each gets its own register allocation), and what they need is
+// read on demand with ds_read.
+#define MK_LDS __attribute__((address_space(3)))
+typedef MK_LDS Smem *SmemPtr;
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef const MK_LDS mk_llama_args &ArgsRef;
+typedef const MK_LDS int *InsPtr;
+
+// value known to be the same in every lane -> scalar register
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+template <class T>
+__device__ __forceinline__ T *uni(T *p) {
+    const uint64_t v = (uint64_t)p;
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+    return (T *)(((uint64_t)hi << 32) | lo);
+}
+
 struct Ctx {
-    const mk_llama_args &a;
-    Smem *sm;
-    int *status;
-    int *shards;
-    int *arrive_o, *arrive_d;
-    float *partial;
+    SmemPtr sm;
     int tid, wave, lane;
     bool controller;
     int worker, slot, opcode;
-    long long spin_ticks;           // wall-clock ticks (100 MHz) a wait may take
-    int barrier_cols;               // H + 2 KVH
     int *trace;                     // this instruction's timing row, or nullptr when tracing is off
-    long long t_launch;             // wall clock when the workgroup started
 };
+
+__device__ __forceinline__ Ctx make_ctx(SmemPtr sm, int slot, int opcode) {
+    ArgsRef a = sm->args;
+    Ctx c;
+    c.sm = sm;
+    c.tid = (int)threadIdx.x;
+    c.wave = c.tid / 64;
+    c.lane = c.tid % 64;
+    c.controller = c.wave == kConsumerWaves;
+    c.worker = (int)blockIdx.x;
+    c.slot = slot;
+    c.opcode = opcode;
+    c.trace = nullptr;
+    if ((a.flags & MK_FLAG_TIMINGS) && a.timings)
+        c.trace = uni(a.timings) + ((size_t)c.worker * uni(a.num_slots) + slot) * MK_TIMING_SLOTS;
+    return c;
+}
+
+// workspace regions
+__device__ __forceinline__ int *ws_ints(const Ctx &c) { return uni(static_cast<int *>(c.sm->args.workspace)); }
+__device__ __forceinline__ WsLayout ws_regions(const Ctx &c) {
+    ArgsRef a = c.sm->args;
+    return ws_layout(uni(a.num_layers), uni(a.hidden_size), uni(a.intermediate_size), uni(a.matvec_reduction_size));
+}
+__device__ __forceinline__ int *ws_status(const Ctx &c) { return ws_ints(c) + ws_regions(c).status; }
+__device__ __forceinline__ int *ws_shards(const Ctx &c) { return ws_ints(c) + ws_regions(c).shards; }
+__device__ __forceinline__ int *ws_arrive(const Ctx &c, bool down) {
+    const WsLayout w = ws_regions(c);
+    return ws_ints(c) + (down ? w.arrive_d : w.arrive_o);
+}
+__device__ __forceinline__ float *ws_partial(const Ctx &c) {
+    return reinterpret_cast<float *>(ws_ints(c) + ws_regions(c).partial);
+}
+__device__ __forceinline__ long long spin_ticks(const Ctx &c) {
+    const uint32_t us = (uint32_t)uni((int)c.sm->args.spin_limit_us);
+    return (long long)(us ? us : 2000000u) * 100;  // 100 MHz wall clock
+}
 
 // Timing slots written per instruction by the controller when MK_FLAG_TIMINGS is set (ticks of
 // the 100 MHz wall clock since the workgroup started; counterpart of the reference's timing
@@ -299,23 +367,33 @@ struct Ctx {
 enum { kEvStart = 0, kEvDepReady = 1, kEvInputReady = 2, kEvComputeDone = 3, kEvEnd = 4, kEvOpcode = 5 };
 
 __device__ __forceinline__ void trace_event(const Ctx &c, int slot) {
-    if (c.trace && c.controller && c.lane == 0) c.trace[slot] = (int)(wall_clock64() - c.t_launch);
+    if (c.trace && c.controller && c.lane == 0) st_plain_i32(c.trace + slot, (int)(wall_clock64() - c.sm->t_launch));
+}
+
+// consumer-side events (wave 0, lane 0), slots 16 and up; for kernel development
+__device__ __forceinline__ void trace_consumer(const Ctx &c, int slot) {
+#ifdef MK_TRACE_CONSUMER
+    if (c.trace && c.tid == 0) st_plain_i32(c.trace + slot, (int)(wall_clock64() - c.sm->t_launch));
+#endif
 }
 
 __device__ __forceinline__ int *bar_ptr(const Ctx &c, int layer, int row, int col) {
-    return c.a.barriers + ((size_t)layer * MK_BARRIER_ROWS + row) * c.barrier_cols + col;
+    ArgsRef a = c.sm->args;
+    const int cols = uni(a.num_attention_heads) + 2 * uni(a.num_kv_heads);
+    return uni(a.barriers) + ((size_t)layer * MK_BARRIER_ROWS + row) * cols + col;
 }
 __device__ __forceinline__ int *shard_ptr(const Ctx &c, int shard, int layer, int row) {
-    return c.shards + ((size_t)shard * c.a.num_layers + layer) * kHotRows + (row - 2);
+    return ws_shards(c) + ((size_t)shard * uni(c.sm->args.num_layers) + layer) * kHotRows + (row - 2);
 }
 
 // first error wins
 __device__ void record_status(const Ctx &c, int code) {
     int expected = 0;
-    if (__hip_atomic_compare_exchange_strong(&c.status[0], &expected, code, __ATOMIC_RELAXED, __ATOMIC_RELAXED, AG)) {
-        st_i32(&c.status[1], c.worker);
-        st_i32(&c.status[2], c.slot);
-        st_i32(&c.status[3], c.opcode);
+    int *status = ws_status(c);
+    if (__hip_atomic_compare_exchange_strong(as_global(&status[0]), &expected, code, __ATOMIC_RELAXED, __ATOMIC_RELAXED, AG)) {
+        st_i32(&status[1], c.worker);
+        st_i32(&status[2], c.slot);
+        st_i32(&status[3], c.opcode);
     }
 }
 
@@ -325,13 +403,15 @@ __device__ void record_status(const Ctx &c, int code) {
 // word so that one worker's failure releases everybody.
 __device__ bool poll_counters(const Ctx &c, const int *ptr, bool sum_mode, int target) {
     const long long t0 = wall_clock64();
+    const long long limit = spin_ticks(c);
+    const int *status = ws_status(c);
     while (true) {
         const int v = ptr ? ld_i32(ptr) : 0;
-        const int st = c.lane == 63 ? ld_i32(c.status) : 0;
+        const int st = c.lane == 63 ? ld_i32(status) : 0;
         const bool ok = sum_mode ? (lane_sum_i32(v) >= target) : (bool)__all(ptr == nullptr || v >= target);
         if (ok) break;
         if (__any(st != 0)) return false;
-        if (wall_clock64() - t0 > c.spin_ticks) {
+        if (wall_clock64() - t0 > limit) {
             if (c.lane == 0) record_status(c, MK_STATUS_BARRIER_TIMEOUT);
             return false;
         }
@@ -409,20 +489,20 @@ __device__ __forceinline__ void rms_norm_x(XVec<KC> &x, const uint16_t *hidden, 
 
 // controller -> consumers hand-over of the activation vector, lane layout
 template <int KC>
-__device__ __forceinline__ void x_to_lds(const XVec<KC> &x, Smem *sm, int lane) {
+__device__ __forceinline__ void x_to_lds(const XVec<KC> &x, SmemPtr sm, int lane) {
 #pragma unroll
     for (int j = 0; j < KC; j++) {
-        float4 *dst = reinterpret_cast<float4 *>(sm->x + (j * 64 + lane) * 8);
-        dst[0] = make_float4(x.v[j][0], x.v[j][1], x.v[j][2], x.v[j][3]);
-        dst[1] = make_float4(x.v[j][4], x.v[j][5], x.v[j][6], x.v[j][7]);
+        MK_LDS f32x4 *dst = (MK_LDS f32x4 *)(sm->x + (j * 64 + lane) * 8);
+        dst[0] = f32x4{x.v[j][0], x.v[j][1], x.v[j][2], x.v[j][3]};
+        dst[1] = f32x4{x.v[j][4], x.v[j][5], x.v[j][6], x.v[j][7]};
     }
 }
 template <int KC>
-__device__ __forceinline__ void x_from_lds(XVec<KC> &x, const Smem *sm, int lane) {
+__device__ __forceinline__ void x_from_lds(XVec<KC> &x, SmemPtr sm, int lane) {
 #pragma unroll
     for (int j = 0; j < KC; j++) {
-        const float4 *src = reinterpret_cast<const float4 *>(sm->x + (j * 64 + lane) * 8);
-        const float4 lo = src[0], hi = src[1];
+        const MK_LDS f32x4 *src = (const MK_LDS f32x4 *)(sm->x + (j * 64 + lane) * 8);
+        const f32x4 lo = src[0], hi = src[1];
         x.v[j][0] = lo.x; x.v[j][1] = lo.y; x.v[j][2] = lo.z; x.v[j][3] = lo.w;
         x.v[j][4] = hi.x; x.v[j][5] = hi.y; x.v[j][6] = hi.z; x.v[j][7] = hi.w;
     }
@@ -476,10 +556,13 @@ __device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need
     }
     const int mine = ntasks > c.wave ? (ntasks - c.wave + kConsumerWaves - 1) / kConsumerWaves : 0;
     uint4 buf[PF][KC];
+    trace_consumer(c, 20);
 #pragma unroll
     for (int s = 0; s < PF; s++)
         if (s < mine) load_row<KC>(buf[s], row_ptr(c.wave + s * kConsumerWaves), c.lane);
+    trace_consumer(c, 21);
     if (!barrier_inputs_ready(c, true)) return false;
+    trace_consumer(c, 22);
     XVec<KC> x;
     if (need_x) x_from_lds<KC>(x, c.sm, c.lane);
     for (int base = 0; base < mine; base += PF) {
@@ -493,6 +576,7 @@ __device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need
             }
         }
     }
+    trace_consumer(c, 23);
     wg_barrier();
 #ifndef MK_NO_EPILOGUE_FIRST
     // hold the next instruction's weight requests back until the controller has sent this
@@ -503,8 +587,9 @@ __device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need
 }
 
 // malformed instruction: every wave evaluates the same condition and leaves; the controller records it
-__device__ __forceinline__ bool bail(const Ctx &c, int code) {
+__device__ __forceinline__ bool bail(const Ctx &c, int code, int *refusal) {
     if (c.controller && c.lane == 0) record_status(c, code);
+    *refusal = code;
     return false;
 }
 
@@ -513,13 +598,15 @@ __device__ __forceinline__ bool bail(const Ctx &c, int code) {
 // reference device op: demos/low-latency-llama/rms_matvec_rope_append.cu:10-231)
 // ---------------------------------------------------------------------------------------------
 template <int KC>
-__device__ __forceinline__ bool op_qkv(const Ctx &c, const int *ins) {
-    const mk_llama_args &a = c.a;
+static __device__ __noinline__ bool op_qkv(SmemPtr lds, int slot, int *refusal) {
+    const InsPtr ins = lds->queue[slot];
+    const Ctx c = make_ctx(lds, slot, ins[0]);
+    ArgsRef a = c.sm->args;
     const int layer = ins[1], start = ins[2], end = ins[3];
     const int hid = a.hidden_size, D = a.head_dim, H = a.num_attention_heads, KVH = a.num_kv_heads;
     const int total_blocks = (H + 2 * KVH) * D / 16;
     if (layer < 0 || layer >= a.num_layers || start < 0 || end > total_blocks || end - start > kOutRows / 16)
-        return bail(c, MK_STATUS_BAD_INSTRUCTION);
+        return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
     const int nblk = end > start ? end - start : 0;
     const uint16_t *W = a.qkv_weights + (size_t)layer * total_blocks * 16 * hid;
     const int down_jobs = (a.intermediate_size / a.matvec_reduction_size) * (hid / 16);
@@ -552,8 +639,8 @@ __device__ __forceinline__ bool op_qkv(const Ctx &c, const int *ins) {
                     const int d = row0 % D;
                     const float *cs = a.rope_cos + (size_t)a.pos_id * D + d;
                     const float *sn = a.rope_sin + (size_t)a.pos_id * D + d;
-                    const float even = (y0 * cs[0]) + ((-y1) * sn[0]);
-                    const float odd = (y1 * cs[1]) + (y0 * sn[1]);
+                    const float even = (y0 * ld_const_f32(cs)) + ((-y1) * ld_const_f32(sn));
+                    const float odd = (y1 * ld_const_f32(cs + 1)) + (y0 * ld_const_f32(sn + 1));
                     packed = mkm::pack_bf16(even, odd);
                 } else {
                     packed = mkm::pack_bf16(y0, y1);
@@ -579,15 +666,17 @@ __device__ __forceinline__ bool op_qkv(const Ctx &c, const int *ins) {
 // rounding chain is reproduced without serialising the workers.
 // ---------------------------------------------------------------------------------------------
 template <int KC>
-__device__ __forceinline__ bool op_matvec_add(const Ctx &c, const int *ins, bool is_down) {
-    const mk_llama_args &a = c.a;
+static __device__ __noinline__ bool op_matvec_add(SmemPtr lds, int slot, bool is_down, int *refusal) {
+    const InsPtr ins = lds->queue[slot];
+    const Ctx c = make_ctx(lds, slot, ins[0]);
+    ArgsRef a = c.sm->args;
     const int layer = ins[1], start = ins[2], end = ins[3], group = ins[4];
     const int hid = a.hidden_size, R = a.matvec_reduction_size;
     const int in_dim = is_down ? a.intermediate_size : hid;
     const int ngroups = in_dim / R;
     if (layer < 0 || layer >= a.num_layers || start < 0 || end > hid / 16 || group < 0 || group >= ngroups ||
         end - start > kOutRows / 16)
-        return bail(c, MK_STATUS_BAD_INSTRUCTION);
+        return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
     const int nblk = end > start ? end - start : 0;
     const uint16_t *W = (is_down ? a.down_weights : a.o_weights) + (size_t)layer * hid * in_dim + (size_t)group * R;
     const uint16_t *vec = (is_down ? a.silu_out : a.attn_out) + (size_t)group * R;
@@ -631,12 +720,13 @@ __device__ __forceinline__ bool op_matvec_add(const Ctx &c, const int *ins, bool
                     st_u32(resid + row0, mkm::pack_bf16(lo, hi));
                 }
             } else {
-                int *arrive = is_down ? c.arrive_d : c.arrive_o;
+                int *arrive = ws_arrive(c, is_down);
+                float *partial = ws_partial(c);
                 for (int t = c.lane; t < nblk * 16; t += 64)
-                    st_f32(c.partial + (size_t)group * hid + start * 16 + t, c.sm->out[t]);
+                    st_f32(partial + (size_t)group * hid + start * 16 + t, c.sm->out[t]);
                 wait_stores();
                 for (int b = c.lane; b < nblk; b += 64) {
-                    const int old = __hip_atomic_fetch_add(&arrive[start + b], 1, __ATOMIC_RELAXED, AG);
+                    const int old = add_ret_i32(&arrive[start + b], 1);
                     const int last = old == ngroups - 1;
                     if (last) st_i32(&arrive[start + b], 0);
                     c.sm->flags[b] = last;
@@ -648,7 +738,7 @@ __device__ __forceinline__ bool op_matvec_add(const Ctx &c, const int *ins, bool
                     const uint32_t h = prefetched ? (p < 64 ? pre[0] : pre[1]) : ld_u32(resid + row0);
                     float lo = mkm::bf16_lo(h), hi = mkm::bf16_hi(h);
                     for (int g = 0; g < ngroups; g++) {
-                        const uint64_t v = ld_u64(c.partial + (size_t)g * hid + row0);
+                        const uint64_t v = ld_u64(partial + (size_t)g * hid + row0);
                         lo = mkm::round_bf16(lo + mkm::bits_f32((uint32_t)v));
                         hi = mkm::round_bf16(hi + mkm::bits_f32((uint32_t)(v >> 32)));
                     }
@@ -665,14 +755,16 @@ __device__ __forceinline__ bool op_matvec_add(const Ctx &c, const int *ins, bool
 // reference device op: demos/low-latency-llama/upgate.cu:10-172)
 // ---------------------------------------------------------------------------------------------
 template <int KC>
-__device__ __forceinline__ bool op_upgate(const Ctx &c, const int *ins) {
-    const mk_llama_args &a = c.a;
+static __device__ __noinline__ bool op_upgate(SmemPtr lds, int slot, int *refusal) {
+    const InsPtr ins = lds->queue[slot];
+    const Ctx c = make_ctx(lds, slot, ins[0]);
+    ArgsRef a = c.sm->args;
     const int layer = ins[1], n = ins[2];
     const int hid = a.hidden_size, inter = a.intermediate_size;
     bool bad = layer < 0 || layer >= a.num_layers || n < 0 || n > MK_INSTRUCTION_WORDS - 3 || n * 32 > kOutRows;
     if (!bad)
         for (int i = 0; i < n; i++) bad |= ins[3 + i] < 0 || ins[3 + i] >= inter / 16;
-    if (bad) return bail(c, MK_STATUS_BAD_INSTRUCTION);
+    if (bad) return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
     const uint16_t *Wu = a.up_weights + (size_t)layer * inter * hid;
     const uint16_t *Wg = a.gate_weights + (size_t)layer * inter * hid;
     const int o_jobs = (hid / a.matvec_reduction_size) * (hid / 16);
@@ -700,7 +792,7 @@ __device__ __forceinline__ bool op_upgate(const Ctx &c, const int *ins) {
         [&]() {
             for (int p = c.lane; p < n * 8; p += 64) {
                 const int i = p >> 3, r = (p & 7) * 2;
-                const float *up = c.sm->out + i * 32, *gate = up + 16;
+                const MK_LDS float *up = c.sm->out + i * 32, *gate = up + 16;
                 // silu(gate) -> bf16, then times up -> bf16 (python_vm.py:161-163)
                 const float s0 = mkm::round_bf16(mkm::silu_exact(gate[r]));
                 const float s1 = mkm::round_bf16(mkm::silu_exact(gate[r + 1]));
@@ -716,11 +808,13 @@ __device__ __forceinline__ bool op_upgate(const Ctx &c, const int *ins) {
 // reference device op: demos/low-latency-llama/rms_lm_head.cu:10-117)
 // ---------------------------------------------------------------------------------------------
 template <int KC>
-__device__ __forceinline__ bool op_lm_head(const Ctx &c, const int *ins) {
-    const mk_llama_args &a = c.a;
+static __device__ __noinline__ bool op_lm_head(SmemPtr lds, int slot, int *refusal) {
+    const InsPtr ins = lds->queue[slot];
+    const Ctx c = make_ctx(lds, slot, ins[0]);
+    ArgsRef a = c.sm->args;
     const int start = ins[1], end = ins[2];
     const int hid = a.hidden_size;
-    if (start < 0 || end > a.vocab_size / 16) return bail(c, MK_STATUS_BAD_INSTRUCTION);
+    if (start < 0 || end > a.vocab_size / 16) return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
     const int down_jobs = (a.intermediate_size / a.matvec_reduction_size) * (hid / 16);
     const int blocks_per_batch = kOutRows / 16;
     bool first = true;
@@ -753,6 +847,24 @@ __device__ __forceinline__ bool op_lm_head(const Ctx &c, const int *ins) {
     return true;
 }
 
+// One level of a recursive-halving tree sum.  `vals` holds N partial sums; the partner is lane
+// (l ^ OFFSET).  The lane whose OFFSET bit is clear keeps the first N/2 entries and sends the second
+// half, the other lane the opposite; afterwards vals[0 .. N/2) holds own + partner for the kept half.
+template <int OFFSET, int N>
+__device__ __forceinline__ void halving_level(float *vals, int lane) {
+    const bool upper = (lane & OFFSET) != 0;
+#pragma unroll
+    for (int k = 0; k < N / 2; k++) {
+        const float keep = upper ? vals[N / 2 + k] : vals[k];
+        const float send = upper ? vals[k] : vals[N / 2 + k];
+        const uint32_t own = __builtin_bit_cast(uint32_t, send);
+        const LanePair pr = lane_xor_pair<OFFSET>(own);
+        // the pair is {own, partner} in unspecified order; if both are equal either will do
+        const uint32_t got = pr.a == own ? pr.b : pr.a;
+        vals[k] = keep + __builtin_bit_cast(float, got);
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // opcode 2: attention of the 4 query heads of one KV head over one partition of the cache
 // (python_vm.py:277-346; reference device op: demos/low-latency-llama/attention_partial.cu).
@@ -763,20 +875,22 @@ __device__ __forceinline__ bool op_lm_head(const Ctx &c, const int *ins) {
 // waves).  Each of the 8 consumer waves plays virtual waves w and w + 8.
 // ---------------------------------------------------------------------------------------------
 template <int D>
-__device__ __forceinline__ bool op_attention(const Ctx &c, const int *ins) {
+static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *refusal) {
+    const InsPtr ins = lds->queue[slot];
+    const Ctx c = make_ctx(lds, slot, ins[0]);
     constexpr int LPT = D / 8;                  // lanes per token
     constexpr int TPW = 64 / LPT;               // tokens per wave per round
     constexpr int NSLOT = kVirtualWaves * TPW;  // tokens per workgroup round
     constexpr int G = kGqa;
     constexpr int VW = kVirtualWaves / kConsumerWaves;  // virtual waves per consumer wave
-    const mk_llama_args &a = c.a;
-    Smem *sm = c.sm;
+    ArgsRef a = c.sm->args;
+    const SmemPtr sm = c.sm;
     const int layer = ins[1], kvh = ins[2], P = ins[3], pidx = ins[4];
     const int H = a.num_attention_heads, KVH = a.num_kv_heads;
     const bool skip = a.skip_attn_reduction != 0;
     if (layer < 0 || layer >= a.num_layers || kvh < 0 || kvh >= KVH || P < 1 || pidx < 0 || pidx >= P ||
         (!skip && pidx >= a.max_partials))
-        return bail(c, MK_STATUS_BAD_INSTRUCTION);
+        return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
     const int seq_len = a.pos_id + 1;
     const int total_blocks = (seq_len + 15) / 16;
     const int bpp = (total_blocks + P - 1) / P;
@@ -785,7 +899,7 @@ __device__ __forceinline__ bool op_attention(const Ctx &c, const int *ins) {
     const int t0 = sb * 16;
     const int t1 = min(eb * 16, seq_len);
     const int T = t1 > t0 ? t1 - t0 : 0;
-    if (T > kScoreCap) return bail(c, MK_STATUS_ATTN_TOO_LONG);
+    if (T > kScoreCap) return bail(c, MK_STATUS_ATTN_TOO_LONG, refusal);
     const int h0 = kvh * G;
     const int rounds = (T + NSLOT - 1) / NSLOT;
 
@@ -827,19 +941,40 @@ __device__ __forceinline__ bool op_attention(const Ctx &c, const int *ins) {
         return t == a.pos_id ? ld_b128(p) : ld_const_b128(p);
     };
 
-    // round 0 of K does not depend on this step except for the newest token: request it early
-    uint4 k0[VW];
+    // Rounds are processed in batches of RU so that RU * VW row loads are in flight per lane.  The
+    // first batch of K does not depend on this step except for the newest token: request it before
+    // the dependency is known.
+    constexpr int RU = 2;
+    uint4 kraw[RU][VW], vraw[RU][VW];
 #pragma unroll
-    for (int v = 0; v < VW; v++) {
-        const int r = token_of(0, v);
-        k0[v] = make_uint4(0, 0, 0, 0);
-        if (r < T && t0 + r != a.pos_id) k0[v] = ld_const_b128(kbase + (size_t)(t0 + r) * tok_stride);
-    }
+    for (int u = 0; u < RU; u++)
+#pragma unroll
+        for (int v = 0; v < VW; v++) {
+            const int r = token_of(u, v);
+            kraw[u][v] = make_uint4(0, 0, 0, 0);
+            if (r < T && t0 + r != a.pos_id) kraw[u][v] = ld_const_b128(kbase + (size_t)(t0 + r) * tok_stride);
+        }
     if (!barrier_inputs_ready(c, true)) return false;
+    trace_consumer(c, 16);
 
     float q[G][8];
+    {
+        uint4 qraw[G];
 #pragma unroll
-    for (int h = 0; h < G; h++) unpack8(ld_b128(a.q_post_rope + (size_t)(h0 + h) * D + sub * 8), q[h]);
+        for (int h = 0; h < G; h++) qraw[h] = ld_b128(a.q_post_rope + (size_t)(h0 + h) * D + sub * 8);
+        // the newest token's K row, if it falls into the first batch
+#pragma unroll
+        for (int u = 0; u < RU; u++)
+#pragma unroll
+            for (int v = 0; v < VW; v++) {
+                const int r = token_of(u, v);
+                if (r < T && t0 + r == a.pos_id) kraw[u][v] = ld_b128(kbase + (size_t)(t0 + r) * tok_stride);
+            }
+#pragma unroll
+        for (int h = 0; h < G; h++) unpack8(qraw[h], q[h]);
+    }
+    if (q[0][0] == 12345.0f) trace_consumer(c, 31);  // forces the loads to have landed
+    trace_consumer(c, 17);
 
     // ---- pass 1: scores and maximum ----
     float mx[VW][G];
@@ -847,32 +982,47 @@ __device__ __forceinline__ bool op_attention(const Ctx &c, const int *ins) {
     for (int v = 0; v < VW; v++)
 #pragma unroll
         for (int h = 0; h < G; h++) mx[v][h] = -INFINITY;
-    for (int rd = 0; rd < rounds; rd++) {
-        uint4 kraw[VW];
+    for (int rb = 0; rb < rounds; rb += RU) {
+        if (rb > 0) {
 #pragma unroll
-        for (int v = 0; v < VW; v++) {
-            const int r = token_of(rd, v);
-            kraw[v] = k0[v];
-            if (r < T && (rd > 0 || t0 + r == a.pos_id)) kraw[v] = load_kv(kbase, r);
+            for (int u = 0; u < RU; u++)
+#pragma unroll
+                for (int v = 0; v < VW; v++) {
+                    const int r = token_of(rb + u, v);
+                    if (r < T) kraw[u][v] = load_kv(kbase, r);
+                }
+        } else {
+            // the first batch of V can be requested now: it is needed right after the maximum
+#pragma unroll
+            for (int u = 0; u < RU; u++)
+#pragma unroll
+                for (int v = 0; v < VW; v++) {
+                    const int r = token_of(u, v);
+                    vraw[u][v] = make_uint4(0, 0, 0, 0);
+                    if (r < T) vraw[u][v] = load_kv(vbase, r);
+                }
         }
 #pragma unroll
-        for (int v = 0; v < VW; v++) {
-            const int r = token_of(rd, v);
-            if (r < T) {  // the LPT lanes of a token share r, so they are active together
-                float kf[8];
-                unpack8(kraw[v], kf);
+        for (int u = 0; u < RU; u++)
 #pragma unroll
-                for (int h = 0; h < G; h++) {
-                    float acc = 0.0f;
+            for (int v = 0; v < VW; v++) {
+                const int r = token_of(rb + u, v);
+                if (r < T) {  // the LPT lanes of a token share r, so they are active together
+                    float kf[8];
+                    unpack8(kraw[u][v], kf);
 #pragma unroll
-                    for (int e = 0; e < 8; e++) acc = fmaf(q[h][e], kf[e], acc);
-                    const float s = group_tree_sum<LPT>(acc) * a.attn_scale;
-                    if (sub == 0) sm->scores[h][r] = s;
-                    mx[v][h] = fmaxf(mx[v][h], s);
+                    for (int h = 0; h < G; h++) {
+                        float acc = 0.0f;
+#pragma unroll
+                        for (int e = 0; e < 8; e++) acc = fmaf(q[h][e], kf[e], acc);
+                        const float s = group_tree_sum<LPT>(acc) * a.attn_scale;
+                        if (sub == 0) sm->scores[h][r] = s;
+                        mx[v][h] = fmaxf(mx[v][h], s);
+                    }
                 }
             }
-        }
     }
+    trace_consumer(c, 18);
 #pragma unroll
     for (int v = 0; v < VW; v++)
 #pragma unroll
@@ -880,6 +1030,7 @@ __device__ __forceinline__ bool op_attention(const Ctx &c, const int *ins) {
             const float m = lane_tree_max<LPT, 64>(mx[v][h]);
             if (c.lane == 0) sm->wave_max[c.wave + v * kConsumerWaves][h] = m;
         }
+    trace_consumer(c, 19);
     wg_barrier();
     float hm[G];
 #pragma unroll
@@ -906,43 +1057,64 @@ __device__ __forceinline__ bool op_attention(const Ctx &c, const int *ins) {
 #pragma unroll
             for (int e = 0; e < 8; e++) acc[v][h][e] = 0.0f;
         }
-    for (int rd = 0; rd < rounds; rd++) {
-        uint4 vraw[VW];
+    for (int rb = 0; rb < rounds; rb += RU) {
+        if (rb > 0) {
 #pragma unroll
-        for (int v = 0; v < VW; v++) {
-            const int r = token_of(rd, v);
-            vraw[v] = make_uint4(0, 0, 0, 0);
-            if (r < T) vraw[v] = load_kv(vbase, r);
+            for (int u = 0; u < RU; u++)
+#pragma unroll
+                for (int v = 0; v < VW; v++) {
+                    const int r = token_of(rb + u, v);
+                    if (r < T) vraw[u][v] = load_kv(vbase, r);
+                }
         }
 #pragma unroll
-        for (int v = 0; v < VW; v++) {
-            const int r = token_of(rd, v);
-            if (r < T) {
-                float vf[8];
-                unpack8(vraw[v], vf);
+        for (int u = 0; u < RU; u++)
 #pragma unroll
-                for (int h = 0; h < G; h++) {
-                    const float p = sm->scores[h][r];
-                    lsum[v][h] = lsum[v][h] + p;
+            for (int v = 0; v < VW; v++) {
+                const int r = token_of(rb + u, v);
+                if (r < T) {
+                    float vf[8];
+                    unpack8(vraw[u][v], vf);
 #pragma unroll
-                    for (int e = 0; e < 8; e++) acc[v][h][e] = fmaf(p, vf[e], acc[v][h][e]);
+                    for (int h = 0; h < G; h++) {
+                        const float p = sm->scores[h][r];
+                        lsum[v][h] = lsum[v][h] + p;
+#pragma unroll
+                        for (int e = 0; e < 8; e++) acc[v][h][e] = fmaf(p, vf[e], acc[v][h][e]);
+                    }
                 }
             }
-        }
     }
-    // combine the TPW slots of each virtual wave (pairwise tree over lane groups), park per wave
+    // Combine the TPW slots of each virtual wave: a pairwise tree over the token groups (lane bits
+    // log2(LPT) .. 5).  Recursive halving: at each level a lane hands half of its partial sums to
+    // its partner and keeps the other half, so the 32 sums per lane shrink to 32 / TPW and the
+    // number of lane exchanges drops from 32 per level to 16 + 8 + 4.  own + partner is the same
+    // addition the butterfly would do.
 #pragma unroll
-    for (int v = 0; v < VW; v++)
+    for (int v = 0; v < VW; v++) {
+        float part[G * 8];
+#pragma unroll
+        for (int h = 0; h < G; h++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) part[h * 8 + e] = acc[v][h][e];
+        halving_level<LPT, G * 8>(part, c.lane);
+        halving_level<LPT * 2, G * 4>(part, c.lane);
+        if constexpr (TPW == 8) halving_level<LPT * 4, G * 2>(part, c.lane);
+        // the lane now holds the sums with index  tg_bit0 * 16 + tg_bit1 * 8 (+ tg_bit2 * 4) + k
+        constexpr int kLeft = G * 8 / TPW;
+        const int first = ((tok_in_wave & 1) * 16) + (((tok_in_wave >> 1) & 1) * 8) + (TPW == 8 ? ((tok_in_wave >> 2) & 1) * 4 : 0);
+        MK_LDS float *dst = &sm->wave_o[c.wave + v * kConsumerWaves][0][0];
+#pragma unroll
+        for (int k = 0; k < kLeft; k++) {
+            const int idx = first + k;  // = h * 8 + e
+            dst[(idx >> 3) * kMaxHeadDim + sub * 8 + (idx & 7)] = part[k];
+        }
 #pragma unroll
         for (int h = 0; h < G; h++) {
             const float l = lane_tree_sum<LPT, 64>(lsum[v][h]);
             if (c.lane == 0) sm->wave_l[c.wave + v * kConsumerWaves][h] = l;
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const float o = lane_tree_sum<LPT, 64>(acc[v][h][e]);
-                if (c.lane < LPT) sm->wave_o[c.wave + v * kConsumerWaves][h][sub * 8 + e] = o;
-            }
         }
+    }
     wg_barrier();
 
     // ---- combine the 16 virtual waves pairwise, normalise, store: thread -> (head, dim pair) ----
@@ -992,9 +1164,11 @@ __device__ __forceinline__ bool op_attention(const Ctx &c, const int *ins) {
 // opcode 3: log-sum-exp merge of attention partitions  (python_vm.py:349-393;
 // reference device op: demos/low-latency-llama/attention_reduction.cu:18-339)
 // ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ bool op_attention_reduction(const Ctx &c, const int *ins) {
-    const mk_llama_args &a = c.a;
-    Smem *sm = c.sm;
+static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot, int *refusal) {
+    const InsPtr ins = lds->queue[slot];
+    const Ctx c = make_ctx(lds, slot, ins[0]);
+    ArgsRef a = c.sm->args;
+    const SmemPtr sm = c.sm;
     const int layer = ins[1], hs = ins[2], P = ins[3], terminal = ins[4], n = ins[5];
     const int D = a.head_dim, R = a.attn_reduction_size, MP = a.max_partials;
     bool bad = layer < 0 || layer >= a.num_layers || n < 1 || n > MK_INSTRUCTION_WORDS - 7 || hs < 0 ||
@@ -1003,19 +1177,27 @@ __device__ __forceinline__ bool op_attention_reduction(const Ctx &c, const int *
         for (int i = 0; i < n; i++) bad |= ins[6 + i] < 0 || ins[6 + i] >= MP;
     const int out_idx = bad ? 0 : ins[6 + n];
     bad |= !terminal && (out_idx < 0 || out_idx >= MP);
-    if (bad) return bail(c, MK_STATUS_BAD_INSTRUCTION);
+    if (bad) return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
 
     if (c.controller) {
         const int *p = c.lane < R ? bar_ptr(c, layer, 1, hs + c.lane) : nullptr;
         const bool ok = poll_counters(c, p, false, P);
         trace_event(c, kEvDepReady);
-        if (ok && c.lane < R) {
-            // weights 2^(lse_i - max) once per (head, list entry)
-            const float *lses = a.attn_lse_intermediates + (size_t)(hs + c.lane) * MP;
-            float m = -INFINITY;
-            for (int i = 0; i < n; i++) m = fmaxf(m, ld_f32(lses + ins[6 + i]));
-            sm->head_m[c.lane] = m;
-            for (int i = 0; i < n; i++) sm->head_w[c.lane][i] = mkm::exp2f_exact(ld_f32(lses + ins[6 + i]) - m);
+        if (ok) {
+            // weights 2^(lse_i - max) once per (head, list entry): lane i takes list entry i, so the
+            // loads of one head go out together
+            float lse[kGqa];
+#pragma unroll
+            for (int h = 0; h < kGqa; h++) {
+                const float *lses = a.attn_lse_intermediates + (size_t)(hs + h) * MP;
+                lse[h] = (h < R && c.lane < n) ? ld_f32(lses + ins[6 + c.lane]) : -INFINITY;
+            }
+#pragma unroll
+            for (int h = 0; h < kGqa; h++) {
+                const float m = lane_tree_max(lse[h]);
+                if (h < R && c.lane < n) sm->head_w[h][c.lane] = mkm::exp2f_exact(lse[h] - m);
+                if (h < R && c.lane == 0) sm->head_m[h] = m;
+            }
         }
         if (!barrier_inputs_ready(c, ok)) return false;
         wg_barrier();  // outputs stored
@@ -1029,12 +1211,21 @@ __device__ __forceinline__ bool op_attention_reduction(const Ctx &c, const int *
         const int head = hs + h;
         const float *outs = a.attn_out_intermediates + (size_t)head * MP * D;
         float den = 0.0f, o0 = 0.0f, o1 = 0.0f;
-        for (int i = 0; i < n; i++) {
-            const float w = sm->head_w[h][i];
-            const uint64_t v = ld_u64(outs + (size_t)ins[6 + i] * D + d);
-            den = den + w;
-            o0 = fmaf(w, mkm::bits_f32((uint32_t)v), o0);
-            o1 = fmaf(w, mkm::bits_f32((uint32_t)(v >> 32)), o1);
+        // accumulate in list order; the loads of up to 13 entries are issued together
+        constexpr int kBatch = 13;
+        for (int i0 = 0; i0 < n; i0 += kBatch) {
+            uint64_t v[kBatch];
+#pragma unroll
+            for (int k = 0; k < kBatch; k++)
+                if (i0 + k < n) v[k] = ld_u64(outs + (size_t)ins[6 + i0 + k] * D + d);
+#pragma unroll
+            for (int k = 0; k < kBatch; k++)
+                if (i0 + k < n) {
+                    const float w = sm->head_w[h][i0 + k];
+                    den = den + w;
+                    o0 = fmaf(w, mkm::bits_f32((uint32_t)v[k]), o0);
+                    o1 = fmaf(w, mkm::bits_f32((uint32_t)(v[k] >> 32)), o1);
+                }
         }
         o0 = o0 / den;
         o1 = o1 / den;
@@ -1059,93 +1250,89 @@ __device__ __forceinline__ bool op_attention_reduction(const Ctx &c, const int *
 template <int KC_HID, int KC_RED, int D>
 __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args a) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
-    Smem *sm = reinterpret_cast<Smem *>(smem_raw);
-    const WsLayout wl = ws_layout(a.num_layers, a.hidden_size, a.intermediate_size, a.matvec_reduction_size);
-    int *ws = static_cast<int *>(a.workspace);
-    Ctx c{a,
-          sm,
-          ws + wl.status,
-          ws + wl.shards,
-          ws + wl.arrive_o,
-          ws + wl.arrive_d,
-          reinterpret_cast<float *>(ws + wl.partial),
-          (int)threadIdx.x,
-          (int)threadIdx.x / 64,
-          (int)threadIdx.x % 64,
-          (int)threadIdx.x / 64 == kConsumerWaves,
-          (int)blockIdx.x,
-          0,
-          0,
-          (long long)(a.spin_limit_us ? a.spin_limit_us : 2000000u) * 100,
-          a.num_attention_heads + 2 * a.num_kv_heads,
-          nullptr,
-          wall_clock64()};
-    const bool tracing = (a.flags & MK_FLAG_TIMINGS) && a.timings;
-    if (c.tid == 0) {
+    const SmemPtr sm = (SmemPtr)smem_raw;
+    const int tid = (int)threadIdx.x;
+    if (tid == 0) {
         sm->abort = 0;
         sm->last_flag = 0;
+        sm->t_launch = wall_clock64();
+    }
+    {
+        // the launch arguments: kernarg segment -> LDS, one word per thread
+        const __attribute__((address_space(4))) int *src =
+            (const __attribute__((address_space(4))) int *)__builtin_amdgcn_kernarg_segment_ptr();
+        MK_LDS int *dst = (MK_LDS int *)&sm->args;
+        static_assert(sizeof(mk_llama_args) % 4 == 0 && sizeof(mk_llama_args) / 4 <= kThreads, "argument block");
+        if (tid < (int)(sizeof(mk_llama_args) / 4)) dst[tid] = src[tid];
     }
     // Instruction fetch (reference: controller warp, include/controller/instruction_fetch.cuh:10-27):
     // the whole queue of this worker is copied into LDS once, so decoding an instruction never
-    // waits on HBM.  Queues longer than the LDS copy are read in place.
-    const int *queue = a.instructions + (size_t)c.worker * a.num_slots * MK_INSTRUCTION_WORDS;
+    // waits on HBM.
     {
-        const int words = min(a.num_slots, kQueueSlots) * MK_INSTRUCTION_WORDS;
-        int *dst = &sm->queue[0][0];
-        for (int i = c.tid; i < words; i += kThreads) dst[i] = queue[i];
+        const int *queue = a.instructions + (size_t)blockIdx.x * a.num_slots * MK_INSTRUCTION_WORDS;
+        const int words = a.num_slots * MK_INSTRUCTION_WORDS;
+        MK_LDS int *dst = &sm->queue[0][0];
+        for (int i = tid; i < words; i += kThreads) dst[i] = queue[i];
     }
     wg_barrier();
 
+    // The handlers get the address of a kernel-local word for their refusal code.  Besides carrying
+    // the code it keeps the calls from being marked as tail calls, which lets the compiler drop the
+    // callee-saved register traffic (dozens of scratch stores and reloads per instruction) from
+    // handlers that only this kernel calls.
+    int refusal = 0;
     for (int slot = 0; slot < a.num_slots; slot++) {
-        const int *ins = slot < kQueueSlots ? sm->queue[slot] : queue + (size_t)slot * MK_INSTRUCTION_WORDS;
-        const int opcode = ins[0];
-        c.slot = slot;
-        c.opcode = opcode;
-        if (tracing) {
-            c.trace = a.timings + ((size_t)c.worker * a.num_slots + slot) * MK_TIMING_SLOTS;
+        const int opcode = sm->queue[slot][0];
+        if (opcode == 0) continue;  // NoOp pads the queues (megakernels/scheduler.py:287-289)
+        {
+            const Ctx c = make_ctx(sm, slot, opcode);
             trace_event(c, kEvStart);
-            if (c.controller && c.lane == 0) c.trace[kEvOpcode] = opcode;
+            if (c.trace && c.controller && c.lane == 0) st_plain_i32(c.trace + kEvOpcode, opcode);
         }
         bool ok = true;
         switch (opcode) {
-        case 0: break;  // NoOp pads the queues (megakernels/scheduler.py:287-289)
-        case 1: ok = op_qkv<KC_HID>(c, ins); break;
-        case 2: ok = op_attention<D>(c, ins); break;
-        case 3: ok = op_attention_reduction(c, ins); break;
-        case 4: ok = op_matvec_add<KC_RED>(c, ins, false); break;
-        case 5: ok = op_upgate<KC_HID>(c, ins); break;
-        case 6: ok = op_matvec_add<KC_RED>(c, ins, true); break;
-        case 7: ok = op_lm_head<KC_HID>(c, ins); break;
-        default: ok = bail(c, MK_STATUS_BAD_OPCODE);  // reference: trap, include/util.cuh:38
+        case 1: ok = op_qkv<KC_HID>(sm, slot, &refusal); break;
+        case 2: ok = op_attention<D>(sm, slot, &refusal); break;
+        case 3: ok = op_attention_reduction(sm, slot, &refusal); break;
+        case 4: ok = op_matvec_add<KC_RED>(sm, slot, false, &refusal); break;
+        case 5: ok = op_upgate<KC_HID>(sm, slot, &refusal); break;
+        case 6: ok = op_matvec_add<KC_RED>(sm, slot, true, &refusal); break;
+        case 7: ok = op_lm_head<KC_HID>(sm, slot, &refusal); break;
+        default: ok = bail(make_ctx(sm, slot, opcode), MK_STATUS_BAD_OPCODE, &refusal);  // reference: trap, include/util.cuh:38
         }
-        trace_event(c, kEvEnd);
+        trace_event(make_ctx(sm, slot, opcode), kEvEnd);
         if (!ok) break;
     }
+    if (refusal && tid == 0) sm->abort = refusal;
 
     // The last workgroup to get here folds the sharded counters into `barriers` and leaves the
     // shards zeroed for the next launch.
     wait_stores();
     wg_barrier();
-    if (c.tid == 0) {
-        const int done = __hip_atomic_fetch_add(&c.status[kDoneSlot], 1, __ATOMIC_RELAXED, AG);
+    const WsLayout wl = ws_layout(a.num_layers, a.hidden_size, a.intermediate_size, a.matvec_reduction_size);
+    int *status = static_cast<int *>(a.workspace) + wl.status;
+    if (tid == 0) {
+        const int done = __hip_atomic_fetch_add(&status[kDoneSlot], 1, __ATOMIC_RELAXED, AG);
         sm->last_flag = done == (int)gridDim.x - 1;
     }
     wg_barrier();
     if (sm->last_flag) {
         const int counters = a.num_layers * kHotRows;
-        for (int i = c.tid; i < counters; i += kThreads) {
+        int *shards = static_cast<int *>(a.workspace) + wl.shards;
+        const int cols = a.num_attention_heads + 2 * a.num_kv_heads;
+        for (int i = tid; i < counters; i += kThreads) {
             int total = 0;
             for (int s = 0; s < kShards; s++) {
-                int *p = c.shards + (size_t)s * counters + i;
+                int *p = shards + (size_t)s * counters + i;
                 const int v = ld_i32(p);
                 if (v) {
                     total += v;
                     st_i32(p, 0);
                 }
             }
-            if (total) add_i32(bar_ptr(c, i / kHotRows, 2 + i % kHotRows, 0), total);
+            if (total) add_i32(a.barriers + ((size_t)(i / kHotRows) * MK_BARRIER_ROWS + 2 + i % kHotRows) * cols, total);
         }
-        if (c.tid == 0) st_i32(&c.status[kDoneSlot], 0);
+        if (tid == 0) st_i32(&status[kDoneSlot], 0);
     }
 }
 
@@ -1239,6 +1426,9 @@ int mk_llama_launch(const mk_llama_args *args, void *hip_stream) {
         return fail(-4, "pos_id %d outside the KV cache (%d) or rope table (%d)", a.pos_id, a.kv_max_len,
                     a.rope_positions);
     if (a.max_partials < 1) return fail(-3, "max_partials must be positive");
+    if (a.num_slots > kQueueSlots)
+        return fail(-3, "instruction queues have %d slots, the kernel keeps at most %d per worker in LDS", a.num_slots,
+                    kQueueSlots);
     KernelFn fn = pick_kernel(hid, R, D);
     if (!fn) return fail(-5, "no kernel instance for hidden %d, reduction width %d, head_dim %d", hid, R, D);
     const uint64_t need = mk_llama_workspace_bytes(a.num_layers, hid, a.intermediate_size, R);
@@ -1278,11 +1468,11 @@ int mk_llama_selftest_bf16(uint64_t *mismatches_out) {
     unsigned long long *dev = nullptr;
     hipError_t e = hipMalloc(&dev, sizeof *dev);
     if (e != hipSuccess) return fail(-9, "hipMalloc: %s", hipGetErrorString(e));
-    hipMemset(dev, 0, sizeof *dev);
+    (void)hipMemset(dev, 0, sizeof *dev);
     hipLaunchKernelGGL(bf16_convert_sweep_kernel, dim3(4096), dim3(256), 0, 0, dev);
     unsigned long long host = 0;
     e = hipMemcpy(&host, dev, sizeof host, hipMemcpyDeviceToHost);
-    hipFree(dev);
+    (void)hipFree(dev);
     if (e != hipSuccess) return fail(-9, "self test: %s", hipGetErrorString(e));
     *mismatches_out = host;
     return 0;
