@@ -28,11 +28,12 @@
 //   * every barrier wait is bounded (spin_limit_us): on expiry the worker records a status
 //     code and every workgroup leaves its instruction loop, so the grid always drains.
 //
-// Arithmetic: bit-compatible with a fixed "lane order" so results can be compared exactly
+// Arithmetic: bit-compatible with a fixed "column order" so results can be compared exactly
 // with a CPU restatement of the Python VM.  A dot product over K elements is computed by one
-// wave: lane l owns elements j*512 + l*8 + e and accumulates them in that order with fmaf,
-// the 64 lane sums are combined by an xor butterfly (a balanced pairwise tree).  Narrowing
-// to bf16 happens exactly where the Python VM narrows (python_vm.py:29-80,127-274).
+// wave: column c = lane * 8 + e accumulates elements j*512 + c in order of j with fmaf (eight
+// independent chains per lane), the 512 column sums are combined as a balanced pairwise tree
+// (within the lane, then an xor butterfly over lanes).  Narrowing to bf16 happens exactly where
+// the Python VM narrows (python_vm.py:29-80,127-274).
 #include <hip/hip_runtime.h>
 
 #include <cstdarg>
@@ -48,7 +49,14 @@ constexpr int kConsumerWaves = 8;
 constexpr int kConsumerThreads = kConsumerWaves * 64;
 constexpr int kThreads = kConsumerThreads + 64;  // + one controller wave
 constexpr int kVirtualWaves = 16;   // attention slot layout is defined for 16 waves; each consumer wave plays two
-constexpr int kShards = 16;         // shards per hot barrier counter
+#ifndef MK_SHARDS
+#define MK_SHARDS 16
+#endif
+#ifndef MK_SHARD_PAD
+#define MK_SHARD_PAD 0
+#endif
+constexpr int kShards = MK_SHARDS;   // shards per hot barrier counter
+constexpr int kShardPad = MK_SHARD_PAD;  // 0: shard-major planes; n > 0: counter-major, n ints per shard
 constexpr int kHotRows = 4;         // barrier rows 2..5 are sharded
 constexpr int kOutRows = 2048;      // rows staged in LDS between matvec and epilogue
 constexpr int kMaxK = 4096;         // longest activation vector handed through LDS
@@ -81,7 +89,8 @@ __host__ __device__ inline WsLayout ws_layout(int L, int hid, int inter, int R) 
     WsLayout w;
     size_t off = 0;
     w.status = off;   off += kStatusInts;
-    w.shards = off;   off += (size_t)kShards * L * kHotRows;
+    off = (off + 31) & ~(size_t)31;  // counters start on a 128-byte line
+    w.shards = off;   off += (size_t)kShards * L * kHotRows * (kShardPad ? kShardPad : 1);
     w.arrive_o = off; off += hid / 16;
     w.arrive_d = off; off += hid / 16;
     off = (off + 3) & ~(size_t)3;
@@ -101,7 +110,10 @@ struct Smem {
     long long t_launch;             // wall clock when the workgroup started
     mk_llama_args args;             // the launch arguments, read from here by every instruction
     int flags[kOutRows / 16];       // per-block "I was the last arriver" (matvec-add)
-    float x[kMaxK];                 // activation vector, lane layout [chunk][lane][8]
+#ifdef MK_TRACE_CONSUMER
+    int consumer_ticks[16];         // development trace: consumer timestamps parked until the instruction ends
+#endif
+    uint32_t x[kMaxK / 2];          // activation vector as bf16 pairs, lane layout [chunk][lane][4 dwords]
     float out[kOutRows];            // matvec row results awaiting the epilogue
     float wave_max[kVirtualWaves][kGqa];
     float wave_l[kVirtualWaves][kGqa];
@@ -154,15 +166,13 @@ __device__ __forceinline__ uint4 ld_const_b128(const void *p) {
 __device__ __forceinline__ float ld_const_f32(const float *p) { return *as_global(p); }
 // plain store of a word nobody else reads during the launch (timing trace)
 __device__ __forceinline__ void st_plain_i32(int *p, int v) { *as_global(p) = v; }
-// weights: read exactly once per step, so stream them past the caches ("nt")
-__device__ __forceinline__ uint4 ld_stream_b128(const void *p) {
+// weights: read exactly once per step, so stream them past the caches (the "nt" bit of the
+// buffer load's cache policy)
 #ifdef MK_NO_NT
-    return ld_const_b128(p);
+#define MK_STREAM_AUX 0
 #else
-    const u32x4 v = __builtin_nontemporal_load(as_global((const u32x4 *)p));
-    return make_uint4(v.x, v.y, v.z, v.w);
+#define MK_STREAM_AUX 2
 #endif
-}
 
 // All of this wave's global stores and atomics have been performed.  The "memory" clobber keeps
 // the compiler from moving memory operations across it.
@@ -373,7 +383,13 @@ __device__ __forceinline__ void trace_event(const Ctx &c, int slot) {
 // consumer-side events (wave 0, lane 0), slots 16 and up; for kernel development
 __device__ __forceinline__ void trace_consumer(const Ctx &c, int slot) {
 #ifdef MK_TRACE_CONSUMER
-    if (c.trace && c.tid == 0) st_plain_i32(c.trace + slot, (int)(wall_clock64() - c.sm->t_launch));
+    if (c.trace && c.tid == 0) c.sm->consumer_ticks[slot - 16] = (int)(wall_clock64() - c.sm->t_launch);
+#endif
+}
+__device__ __forceinline__ void trace_consumer_flush(const Ctx &c, int first, int last) {
+#ifdef MK_TRACE_CONSUMER
+    if (c.trace && c.tid == 0)
+        for (int s = first; s <= last; s++) st_plain_i32(c.trace + s, c.sm->consumer_ticks[s - 16]);
 #endif
 }
 
@@ -383,6 +399,7 @@ __device__ __forceinline__ int *bar_ptr(const Ctx &c, int layer, int row, int co
     return uni(a.barriers) + ((size_t)layer * MK_BARRIER_ROWS + row) * cols + col;
 }
 __device__ __forceinline__ int *shard_ptr(const Ctx &c, int shard, int layer, int row) {
+    if (kShardPad) return ws_shards(c) + ((size_t)(layer * kHotRows + (row - 2)) * kShards + shard) * kShardPad;
     return ws_shards(c) + ((size_t)shard * uni(c.sm->args.num_layers) + layer) * kHotRows + (row - 2);
 }
 
@@ -466,69 +483,112 @@ __device__ __forceinline__ void load_x(XVec<KC> &x, const uint16_t *src, int lan
     for (int j = 0; j < KC; j++) unpack8(raw[j], x.v[j]);
 }
 
-// python_vm.py:50-56: w * bf16(x * rsqrt(mean(x^2) + eps)), statistics in fp32
+// Sum of the 8 per-lane column accumulators, pairwise in column order.
+__device__ __forceinline__ float fold8(const float (&a)[8]) {
+    return ((a[0] + a[1]) + (a[2] + a[3])) + ((a[4] + a[5]) + (a[6] + a[7]));
+}
+
+// python_vm.py:50-56: w * bf16(x * rsqrt(mean(x^2) + eps)), statistics in fp32.  Result as bf16 pairs.
+// Sum of squares in column order: column c = lane * 8 + e accumulates its elements j * 512 + c in
+// order of j, the 512 columns are added as a balanced pairwise tree.
 template <int KC>
-__device__ __forceinline__ void rms_norm_x(XVec<KC> &x, const uint16_t *hidden, const uint4 (&wraw)[KC], float eps,
+__device__ __forceinline__ void rms_norm_x(uint4 (&xq)[KC], const uint16_t *hidden, const uint4 (&wraw)[KC], float eps,
                                            int lane) {
+    XVec<KC> x;
     load_x<KC>(x, hidden, lane);
-    float acc = 0.0f;
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
     for (int j = 0; j < KC; j++)
 #pragma unroll
-        for (int e = 0; e < 8; e++) acc = fmaf(x.v[j][e], x.v[j][e], acc);
-    const float mean = wave_tree_sum_uniform(acc) / (float)(KC * 512);
+        for (int e = 0; e < 8; e++) acc[e] = fmaf(x.v[j][e], x.v[j][e], acc[e]);
+    const float mean = wave_tree_sum_uniform(fold8(acc)) / (float)(KC * 512);
     const float inv = 1.0f / sqrtf(mean + eps);
 #pragma unroll
     for (int j = 0; j < KC; j++) {
-        float wv[8];
+        float wv[8], y[8];
         unpack8(wraw[j], wv);
 #pragma unroll
-        for (int e = 0; e < 8; e++) x.v[j][e] = mkm::round_bf16(wv[e] * mkm::round_bf16(x.v[j][e] * inv));
+        for (int e = 0; e < 8; e++) y[e] = wv[e] * mkm::round_bf16(x.v[j][e] * inv);
+        xq[j].x = mkm::pack_bf16(y[0], y[1]);
+        xq[j].y = mkm::pack_bf16(y[2], y[3]);
+        xq[j].z = mkm::pack_bf16(y[4], y[5]);
+        xq[j].w = mkm::pack_bf16(y[6], y[7]);
     }
 }
 
-// controller -> consumers hand-over of the activation vector, lane layout
+// activation vector written earlier in this launch by other CUs, kept as bf16 pairs
 template <int KC>
-__device__ __forceinline__ void x_to_lds(const XVec<KC> &x, SmemPtr sm, int lane) {
+__device__ __forceinline__ void load_xq(uint4 (&xq)[KC], const uint16_t *src, int lane) {
 #pragma unroll
-    for (int j = 0; j < KC; j++) {
-        MK_LDS f32x4 *dst = (MK_LDS f32x4 *)(sm->x + (j * 64 + lane) * 8);
-        dst[0] = f32x4{x.v[j][0], x.v[j][1], x.v[j][2], x.v[j][3]};
-        dst[1] = f32x4{x.v[j][4], x.v[j][5], x.v[j][6], x.v[j][7]};
-    }
+    for (int j = 0; j < KC; j++) xq[j] = ld_b128(src + j * 512 + lane * 8);
+}
+
+// controller -> consumers hand-over of the activation vector: each lane's 16 bytes of a chunk are
+// adjacent to its neighbours', so the 128-bit LDS accesses are free of bank conflicts
+template <int KC>
+__device__ __forceinline__ void x_to_lds(const uint4 (&xq)[KC], SmemPtr sm, int lane) {
+#pragma unroll
+    for (int j = 0; j < KC; j++)
+        *(MK_LDS u32x4 *)(sm->x + (j * 64 + lane) * 4) = u32x4{xq[j].x, xq[j].y, xq[j].z, xq[j].w};
 }
 template <int KC>
 __device__ __forceinline__ void x_from_lds(XVec<KC> &x, SmemPtr sm, int lane) {
 #pragma unroll
     for (int j = 0; j < KC; j++) {
-        const MK_LDS f32x4 *src = (const MK_LDS f32x4 *)(sm->x + (j * 64 + lane) * 8);
-        const f32x4 lo = src[0], hi = src[1];
-        x.v[j][0] = lo.x; x.v[j][1] = lo.y; x.v[j][2] = lo.z; x.v[j][3] = lo.w;
-        x.v[j][4] = hi.x; x.v[j][5] = hi.y; x.v[j][6] = hi.z; x.v[j][7] = hi.w;
+        const u32x4 r = *(const MK_LDS u32x4 *)(sm->x + (j * 64 + lane) * 4);
+        unpack8(uint4{r.x, r.y, r.z, r.w}, x.v[j]);
     }
 }
 
+// A weight row of an instruction: a buffer resource (uniform) and the row's byte offset in it.
+struct WeightBuffer {
+    const uint16_t *base;
+    uint32_t bytes;
+};
+struct RowRef {
+    WeightBuffer buffer;
+    uint32_t offset;
+};
+__device__ __forceinline__ WeightBuffer weight_buffer(const uint16_t *base, size_t bytes) {
+    return WeightBuffer{uni(base), (uint32_t)uni((int)bytes)};
+}
+constexpr uint32_t kNoRow = 0x80000000u;  // beyond any buffer: the load returns zeros and fetches nothing
+
+// Request one row (KC x 16 bytes per lane), streaming.  `valid` false turns the request into a no-op
+// that still counts as KC loads, which keeps the number of outstanding loads independent of the data.
+template <int KC>
+__device__ __forceinline__ void load_row(uint4 (&w)[KC], const RowRef &r, bool valid, int lane) {
+    const uint32_t off = valid ? r.offset + lane * 16 : kNoRow;
+    // the descriptor lives in scalar registers; which buffer a row comes from is the same for the
+    // whole wave, and readfirstlane says so
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)uni(r.buffer.base), 0, uni((int)r.buffer.bytes), 0x00020000);
+#pragma unroll
+    for (int j = 0; j < KC; j++) {
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, j * 1024, MK_STREAM_AUX);
+        w[j] = uint4{v.x, v.y, v.z, v.w};
+    }
+}
+// plain row load for the small per-instruction vectors (norm weights)
 template <int KC>
 __device__ __forceinline__ void load_row(uint4 (&w)[KC], const uint16_t *row, int lane) {
 #pragma unroll
-    for (int j = 0; j < KC; j++) w[j] = ld_stream_b128(row + j * 512 + lane * 8);
+    for (int j = 0; j < KC; j++) w[j] = ld_const_b128(row + j * 512 + lane * 8);
 }
 
+// dot(w, x) in column order: column c = lane * 8 + e accumulates w[j*512+c] * x[j*512+c] over j with
+// fused multiply-add from 0; the 512 columns are added as a balanced pairwise tree.
 template <int KC>
 __device__ __forceinline__ float dot_row(const uint4 (&w)[KC], const XVec<KC> &x) {
-    float acc = 0.0f;
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
     for (int j = 0; j < KC; j++) {
-        acc = fmaf(mkm::bf16_lo(w[j].x), x.v[j][0], acc);
-        acc = fmaf(mkm::bf16_hi(w[j].x), x.v[j][1], acc);
-        acc = fmaf(mkm::bf16_lo(w[j].y), x.v[j][2], acc);
-        acc = fmaf(mkm::bf16_hi(w[j].y), x.v[j][3], acc);
-        acc = fmaf(mkm::bf16_lo(w[j].z), x.v[j][4], acc);
-        acc = fmaf(mkm::bf16_hi(w[j].z), x.v[j][5], acc);
-        acc = fmaf(mkm::bf16_lo(w[j].w), x.v[j][6], acc);
-        acc = fmaf(mkm::bf16_hi(w[j].w), x.v[j][7], acc);
+        float wv[8];
+        unpack8(w[j], wv);
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] = fmaf(wv[e], x.v[j][e], acc[e]);
     }
-    return wave_tree_sum_uniform(acc);
+    return wave_tree_sum_uniform(fold8(acc));
 }
 
 // One batch of a matvec instruction.
@@ -537,8 +597,8 @@ __device__ __forceinline__ float dot_row(const uint4 (&w)[KC], const XVec<KC> &x
 //   controller: `prepare` (wait for the dependency, build the activation vector in LDS; returns
 //               false to abandon), barrier, `overlap`, barrier, `finish` (epilogue + signal)
 // Both barriers are reached by all nine waves whatever the outcome of `prepare`.
-template <int KC, class RowPtr, class Prepare, class Overlap, class Finish>
-__device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need_x, RowPtr row_ptr, Prepare prepare,
+template <int KC, class RowOf, class Prepare, class Overlap, class Finish>
+__device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need_x, RowOf row_ref, Prepare prepare,
                                              Overlap overlap, Finish finish) {
     constexpr int PF = rows_in_flight<KC>();
     if (c.controller) {
@@ -556,28 +616,38 @@ __device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need
     }
     const int mine = ntasks > c.wave ? (ntasks - c.wave + kConsumerWaves - 1) / kConsumerWaves : 0;
     uint4 buf[PF][KC];
+    // Every request below is issued unconditionally (rows past the end are no-op requests), so the
+    // count of outstanding loads at each wait is a compile-time constant: the wait for row i leaves
+    // the PF - 1 younger rows in flight.
+    auto request = [&](uint4 (&dst)[KC], int i) {
+        const bool valid = i < mine;
+        load_row<KC>(dst, row_ref(valid ? c.wave + i * kConsumerWaves : 0), valid, c.lane);
+    };
     trace_consumer(c, 20);
 #pragma unroll
-    for (int s = 0; s < PF; s++)
-        if (s < mine) load_row<KC>(buf[s], row_ptr(c.wave + s * kConsumerWaves), c.lane);
+    for (int s = 0; s < PF; s++) request(buf[s], s);
     trace_consumer(c, 21);
     if (!barrier_inputs_ready(c, true)) return false;
     trace_consumer(c, 22);
     XVec<KC> x;
     if (need_x) x_from_lds<KC>(x, c.sm, c.lane);
+    trace_consumer(c, 24);
     for (int base = 0; base < mine; base += PF) {
+        if (base == PF) trace_consumer(c, 25);
 #pragma unroll
         for (int s = 0; s < PF; s++) {
             const int i = base + s;
-            if (i < mine) {
-                const float y = mkm::round_bf16(dot_row<KC>(buf[s], x));
-                if (i + PF < mine) load_row<KC>(buf[s], row_ptr(c.wave + (i + PF) * kConsumerWaves), c.lane);
-                if (c.lane == 0) c.sm->out[c.wave + i * kConsumerWaves] = y;
-            }
+            float y = 0.0f;
+            if (i < mine) y = mkm::round_bf16(dot_row<KC>(buf[s], x));
+            compiler_fence();
+            request(buf[s], i + PF);
+            compiler_fence();
+            if (i < mine && c.lane == 0) c.sm->out[c.wave + i * kConsumerWaves] = y;
         }
     }
     trace_consumer(c, 23);
     wg_barrier();
+    trace_consumer_flush(c, 20, 25);
 #ifndef MK_NO_EPILOGUE_FIRST
     // hold the next instruction's weight requests back until the controller has sent this
     // instruction's results and signal: they would otherwise queue behind the bulk loads
@@ -608,20 +678,21 @@ static __device__ __noinline__ bool op_qkv(SmemPtr lds, int slot, int *refusal) 
     if (layer < 0 || layer >= a.num_layers || start < 0 || end > total_blocks || end - start > kOutRows / 16)
         return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
     const int nblk = end > start ? end - start : 0;
-    const uint16_t *W = a.qkv_weights + (size_t)layer * total_blocks * 16 * hid;
+    const size_t matrix_bytes = (size_t)total_blocks * 16 * hid * 2;
+    const WeightBuffer W = weight_buffer(a.qkv_weights + (size_t)layer * total_blocks * 16 * hid, matrix_bytes);
     const int down_jobs = (a.intermediate_size / a.matvec_reduction_size) * (hid / 16);
 
     return matvec_batch<KC>(
-        c, nblk * 16, nblk > 0, [&](int t) { return W + (size_t)(start * 16 + t) * hid; },
+        c, nblk * 16, nblk > 0, [&](int t) { return RowRef{W, (uint32_t)(start * 16 + t) * (uint32_t)hid * 2u}; },
         [&]() {
             uint4 wraw[KC];
             if (nblk > 0) load_row<KC>(wraw, a.attn_norm_weights + (size_t)layer * hid, c.lane);
             if (layer > 0 && !poll_sharded(c, layer - 1, 5, down_jobs)) return false;
             trace_event(c, kEvDepReady);
             if (nblk > 0) {
-                XVec<KC> x;
-                rms_norm_x<KC>(x, a.hidden_states, wraw, a.rms_norm_eps, c.lane);
-                x_to_lds<KC>(x, c.sm, c.lane);
+                uint4 xq[KC];
+                rms_norm_x<KC>(xq, a.hidden_states, wraw, a.rms_norm_eps, c.lane);
+                x_to_lds<KC>(xq, c.sm, c.lane);
             }
             return true;
         },
@@ -678,7 +749,10 @@ static __device__ __noinline__ bool op_matvec_add(SmemPtr lds, int slot, bool is
         end - start > kOutRows / 16)
         return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
     const int nblk = end > start ? end - start : 0;
-    const uint16_t *W = (is_down ? a.down_weights : a.o_weights) + (size_t)layer * hid * in_dim + (size_t)group * R;
+    // the buffer starts at this column group's first element of the layer's matrix
+    const WeightBuffer W =
+        weight_buffer((is_down ? a.down_weights : a.o_weights) + (size_t)layer * hid * in_dim + (size_t)group * R,
+                      ((size_t)(hid - 1) * in_dim + R) * 2);
     const uint16_t *vec = (is_down ? a.silu_out : a.attn_out) + (size_t)group * R;
     const int wait_row = is_down ? 4 : 2;
     const int wait_target = is_down ? a.intermediate_size / 16 : a.num_attention_heads;
@@ -690,14 +764,14 @@ static __device__ __noinline__ bool op_matvec_add(SmemPtr lds, int slot, bool is
     const bool prefetched = nblk * 8 <= kPre * 64;
 
     return matvec_batch<KC>(
-        c, nblk * 16, nblk > 0, [&](int t) { return W + (size_t)(start * 16 + t) * in_dim; },
+        c, nblk * 16, nblk > 0, [&](int t) { return RowRef{W, (uint32_t)(start * 16 + t) * (uint32_t)in_dim * 2u}; },
         [&]() {
             if (!poll_sharded(c, layer, wait_row, wait_target)) return false;
             trace_event(c, kEvDepReady);
             if (nblk > 0) {
-                XVec<KC> x;
-                load_x<KC>(x, vec, c.lane);
-                x_to_lds<KC>(x, c.sm, c.lane);
+                uint4 xq[KC];
+                load_xq<KC>(xq, vec, c.lane);
+                x_to_lds<KC>(xq, c.sm, c.lane);
             }
             return true;
         },
@@ -765,8 +839,9 @@ static __device__ __noinline__ bool op_upgate(SmemPtr lds, int slot, int *refusa
     if (!bad)
         for (int i = 0; i < n; i++) bad |= ins[3 + i] < 0 || ins[3 + i] >= inter / 16;
     if (bad) return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
-    const uint16_t *Wu = a.up_weights + (size_t)layer * inter * hid;
-    const uint16_t *Wg = a.gate_weights + (size_t)layer * inter * hid;
+    const size_t matrix_bytes = (size_t)inter * hid * 2;
+    const WeightBuffer Wu = weight_buffer(a.up_weights + (size_t)layer * inter * hid, matrix_bytes);
+    const WeightBuffer Wg = weight_buffer(a.gate_weights + (size_t)layer * inter * hid, matrix_bytes);
     const int o_jobs = (hid / a.matvec_reduction_size) * (hid / 16);
 
     // task t: list entry t / 32, matrix (t / 16) & 1 (0 up, 1 gate), row t % 16
@@ -774,7 +849,7 @@ static __device__ __noinline__ bool op_upgate(SmemPtr lds, int slot, int *refusa
         c, n * 32, n > 0,
         [&](int t) {
             const int blk = ins[3 + (t >> 5)];
-            return ((t >> 4) & 1 ? Wg : Wu) + (size_t)(blk * 16 + (t & 15)) * hid;
+            return RowRef{(t >> 4) & 1 ? Wg : Wu, (uint32_t)(blk * 16 + (t & 15)) * (uint32_t)hid * 2u};
         },
         [&]() {
             uint4 wraw[KC];
@@ -782,9 +857,9 @@ static __device__ __noinline__ bool op_upgate(SmemPtr lds, int slot, int *refusa
             if (!poll_sharded(c, layer, 3, o_jobs)) return false;
             trace_event(c, kEvDepReady);
             if (n > 0) {
-                XVec<KC> x;
-                rms_norm_x<KC>(x, a.hidden_states, wraw, a.rms_norm_eps, c.lane);
-                x_to_lds<KC>(x, c.sm, c.lane);
+                uint4 xq[KC];
+                rms_norm_x<KC>(xq, a.hidden_states, wraw, a.rms_norm_eps, c.lane);
+                x_to_lds<KC>(xq, c.sm, c.lane);
             }
             return true;
         },
@@ -817,22 +892,23 @@ static __device__ __noinline__ bool op_lm_head(SmemPtr lds, int slot, int *refus
     if (start < 0 || end > a.vocab_size / 16) return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
     const int down_jobs = (a.intermediate_size / a.matvec_reduction_size) * (hid / 16);
     const int blocks_per_batch = kOutRows / 16;
+    const WeightBuffer W = weight_buffer(a.lm_head_weights, (size_t)a.vocab_size * hid * 2);
     bool first = true;
     int b0 = start;
     do {
         const int b1 = min(b0 + blocks_per_batch, end);
         const int nblk = b1 > b0 ? b1 - b0 : 0;
         const bool ok = matvec_batch<KC>(
-            c, nblk * 16, true, [&](int t) { return a.lm_head_weights + (size_t)(b0 * 16 + t) * hid; },
+            c, nblk * 16, true, [&](int t) { return RowRef{W, (uint32_t)(b0 * 16 + t) * (uint32_t)hid * 2u}; },
             [&]() {
                 if (!first) return true;  // the activation vector stays in LDS between batches
                 uint4 wraw[KC];
                 load_row<KC>(wraw, a.lm_head_norm_weights, c.lane);
                 if (!poll_sharded(c, a.num_layers - 1, 5, down_jobs)) return false;
                 trace_event(c, kEvDepReady);
-                XVec<KC> x;
-                rms_norm_x<KC>(x, a.hidden_states, wraw, a.rms_norm_eps, c.lane);
-                x_to_lds<KC>(x, c.sm, c.lane);
+                uint4 xq[KC];
+                rms_norm_x<KC>(xq, a.hidden_states, wraw, a.rms_norm_eps, c.lane);
+                x_to_lds<KC>(xq, c.sm, c.lane);
                 return true;
             },
             [&]() {},
@@ -1032,6 +1108,7 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
         }
     trace_consumer(c, 19);
     wg_barrier();
+    trace_consumer_flush(c, 16, 19);
     float hm[G];
 #pragma unroll
     for (int h = 0; h < G; h++) {
@@ -1323,7 +1400,7 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
         for (int i = tid; i < counters; i += kThreads) {
             int total = 0;
             for (int s = 0; s < kShards; s++) {
-                int *p = shards + (size_t)s * counters + i;
+                int *p = kShardPad ? shards + ((size_t)i * kShards + s) * kShardPad : shards + (size_t)s * counters + i;
                 const int v = ld_i32(p);
                 if (v) {
                     total += v;
@@ -1426,6 +1503,9 @@ int mk_llama_launch(const mk_llama_args *args, void *hip_stream) {
         return fail(-4, "pos_id %d outside the KV cache (%d) or rope table (%d)", a.pos_id, a.kv_max_len,
                     a.rope_positions);
     if (a.max_partials < 1) return fail(-3, "max_partials must be positive");
+    // weight rows are addressed as 32-bit offsets into one buffer per matrix
+    const uint64_t widest = 2ull * hid * (uint64_t)(a.vocab_size > a.intermediate_size ? a.vocab_size : a.intermediate_size);
+    if (widest >= (1ull << 31)) return fail(-3, "a weight matrix of %llu bytes exceeds the 2 GiB a buffer can address", (unsigned long long)widest);
     if (a.num_slots > kQueueSlots)
         return fail(-3, "instruction queues have %d slots, the kernel keeps at most %d per worker in LDS", a.num_slots,
                     kQueueSlots);

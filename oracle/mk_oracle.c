@@ -26,12 +26,15 @@
  *   residual add  bf16 + bf16 -> bf16, partial sums applied in instruction order   (:59-80)
  *   attention     fp32 throughout; bf16 only when written to attn_out              (:316-330)
  *
- * Canonical summation order ("lane order"):
- *   dot product over K elements (K a multiple of 512): 64 lanes; lane l owns
- *   elements j*512 + l*8 + e (j = 0..K/512-1, e = 0..7) and accumulates them in
- *   that order with fused multiply-add starting from 0; the 64 lane sums are
- *   then added pairwise as a balanced binary tree in lane-index order
- *   ((0+1)+(2+3))+... .  A head-dimension dot product uses D/8 lanes the same way.
+ * Canonical summation order ("column order"):
+ *   dot product over K elements (K a multiple of 512): 512 column accumulators;
+ *   column c accumulates elements j*512 + c (j = 0..K/512-1) in order of j with
+ *   fused multiply-add starting from 0; the 512 column sums are then added
+ *   pairwise as a balanced binary tree in column-index order ((0+1)+(2+3))+... .
+ *   The sum of squares of the RMS norm is formed the same way.
+ *   A head-dimension dot product uses D/8 lanes; lane l accumulates its elements
+ *   l*8 .. l*8+7 in order with fused multiply-add and the lanes are added as a
+ *   balanced binary tree.
  *   Attention over a token range: relative token r goes to slot r mod NSLOT
  *   (NSLOT = 8192/D); each slot accumulates its tokens in increasing order
  *   (fused multiply-add for p*v, plain add for the denominator); the slots
@@ -91,32 +94,25 @@ static float tree_sum(float *v, int n) { /* n a power of two; destroys v */
     return v[0];
 }
 
-/* dot(w[0..K), x[0..K)), w bf16, x fp32, lane order */
+/* dot(w[0..K), x[0..K)), w bf16, x fp32, column order */
 static float dot_lanes(const uint16_t *w, const float *x, int K) {
-    float acc[64];
-    for (int l = 0; l < 64; l++) acc[l] = 0.0f;
+    float acc[512];
+    for (int c = 0; c < 512; c++) acc[c] = 0.0f;
     for (int j = 0; j < K; j += 512)
-        for (int l = 0; l < 64; l++) {
-            const uint16_t *wp = w + j + l * 8;
-            const float *xp = x + j + l * 8;
-            float a = acc[l];
-            for (int e = 0; e < 8; e++) a = fmaf(orc_bf16_to_f32(wp[e]), xp[e], a);
-            acc[l] = a;
-        }
-    return tree_sum(acc, 64);
+        for (int c = 0; c < 512; c++) acc[c] = fmaf(orc_bf16_to_f32(w[j + c]), x[j + c], acc[c]);
+    return tree_sum(acc, 512);
 }
 
 /* python_vm.py:50-56.  out[i] = float(bf16(w[i] * bf16(x[i] * rsqrt(mean(x^2) + eps)))) */
 static void rms_norm(const uint16_t *x, const uint16_t *w, float eps, int n, float *out) {
-    float acc[64];
-    for (int l = 0; l < 64; l++) acc[l] = 0.0f;
+    float acc[512];
+    for (int c = 0; c < 512; c++) acc[c] = 0.0f;
     for (int j = 0; j < n; j += 512)
-        for (int l = 0; l < 64; l++)
-            for (int e = 0; e < 8; e++) {
-                float v = orc_bf16_to_f32(x[j + l * 8 + e]);
-                acc[l] = fmaf(v, v, acc[l]);
-            }
-    float mean = tree_sum(acc, 64) / (float)n;
+        for (int c = 0; c < 512; c++) {
+            float v = orc_bf16_to_f32(x[j + c]);
+            acc[c] = fmaf(v, v, acc[c]);
+        }
+    float mean = tree_sum(acc, 512) / (float)n;
     float inv = 1.0f / sqrtf(mean + eps);
     for (int i = 0; i < n; i++) {
         float normed = orc_round_bf16(orc_bf16_to_f32(x[i]) * inv);

@@ -99,7 +99,7 @@ def test_exp_exp2_log2_accuracy():
     assert lib.mk_oracle_log2f(8.0) == 3.0 and lib.mk_oracle_log2f(1.0) == 0.0
 
 
-def test_dot_lane_order():
+def test_dot_column_order():
     lib = pyvm.load_lib()
     rng = np.random.default_rng(1)
     for K in (512, 2048, 4096):
@@ -109,20 +109,19 @@ def test_dot_lane_order():
         got = lib.mk_oracle_dot(ctypes.cast(w.data_ptr(), pyvm._U16P), ctypes.cast(x.data_ptr(), pyvm._F32P), K)
         want = float(f64(w) @ f64(x))
         assert abs(got - want) <= 1e-5 * math.sqrt(K) * 4
-        # the documented order: lane l owns elements j*512 + l*8 + e, then a pairwise tree over lanes
-        acc = np.zeros(64, dtype=np.float64)
+        # the documented order: column c accumulates elements j*512 + c in order of j, then a
+        # pairwise tree over the 512 columns
         wf, xf = w.float().numpy(), x.numpy()
-        lanes = np.zeros(64, dtype=np.float32)
-        for l in range(64):
+        lanes = np.zeros(512, dtype=np.float32)
+        for col in range(512):
             a = np.float32(0)
             for j in range(0, K, 512):
-                for e in range(8):
-                    k = j + l * 8 + e
-                    a = np.float32(math.fma(float(wf[k]), float(xf[k]), float(a))) if hasattr(math, "fma") else np.float32(np.float64(wf[k]) * np.float64(xf[k]) + np.float64(a))
-                lanes[l] = a
+                k = j + col
+                a = np.float32(math.fma(float(wf[k]), float(xf[k]), float(a))) if hasattr(math, "fma") else np.float32(np.float64(wf[k]) * np.float64(xf[k]) + np.float64(a))
+            lanes[col] = a
         s = 1
-        while s < 64:
-            for i in range(0, 64, 2 * s):
+        while s < 512:
+            for i in range(0, 512, 2 * s):
                 lanes[i] = np.float32(lanes[i] + lanes[i + s])
             s *= 2
         # a float64 multiply-add rounded once to float32 is a fused multiply-add for bf16 x fp32
