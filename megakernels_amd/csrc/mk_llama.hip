@@ -67,14 +67,27 @@ constexpr int kGqa = 4;             // query heads per KV head handled by one at
 constexpr int kStatusInts = 16;
 constexpr int kDoneSlot = 8;        // workspace int: workgroups finished
 
-// Weight rows in flight per consumer wave (16 VGPRs per 2048-element row; the 9-wave workgroup
-// leaves each lane 168 VGPRs).  8 waves x 3 rows x 4 KB = 96 KB per CU; measured on MI355X, 2, 3, 4
-// and 6 rows stream equally fast, and deeper queues only delay the controller's small loads.
-#ifndef MK_ROWS_IN_FLIGHT
-#define MK_ROWS_IN_FLIGHT 3
+// Weight rows in flight per consumer wave, per instruction kind (16 VGPRs per 2048-element row; the
+// 9-wave workgroup leaves each lane 168 VGPRs).  The rows requested before the dependency wait are
+// the prefetch; rows a wave does not have become no-op requests, so the depth follows the rows per
+// wave of the usual schedules: QKV 2, O-proj 1, up/gate 8, down 4.
+#ifndef MK_PF_QKV
+#define MK_PF_QKV 2
+#endif
+#ifndef MK_PF_OPROJ
+#define MK_PF_OPROJ 2
+#endif
+#ifndef MK_PF_UPGATE
+#define MK_PF_UPGATE 4
+#endif
+#ifndef MK_PF_DOWN
+#define MK_PF_DOWN 4
+#endif
+#ifndef MK_PF_LMHEAD
+#define MK_PF_LMHEAD 4
 #endif
 template <int KC>
-constexpr int rows_in_flight() { return KC <= 4 ? MK_ROWS_IN_FLIGHT : 2; }
+constexpr int rows_in_flight(int wanted) { return KC <= 4 ? wanted : (wanted < 2 ? wanted : 2); }
 
 #define AG __HIP_MEMORY_SCOPE_AGENT
 
@@ -555,7 +568,10 @@ __device__ __forceinline__ WeightBuffer weight_buffer(const uint16_t *base, size
 constexpr uint32_t kNoRow = 0x80000000u;  // beyond any buffer: the load returns zeros and fetches nothing
 
 // Request one row (KC x 16 bytes per lane), streaming.  `valid` false turns the request into a no-op
-// that still counts as KC loads, which keeps the number of outstanding loads independent of the data.
+// that still counts as KC loads, which keeps the number of outstanding loads independent of the
+// data: every lane asks for an address beyond the buffer, which returns zeros and fetches nothing.
+// A no-op is not free (it occupies the CU's address path like a real row), so the callers arrange
+// for few of them.
 template <int KC>
 __device__ __forceinline__ void load_row(uint4 (&w)[KC], const RowRef &r, bool valid, int lane) {
     const uint32_t off = valid ? r.offset + lane * 16 : kNoRow;
@@ -597,10 +613,9 @@ __device__ __forceinline__ float dot_row(const uint4 (&w)[KC], const XVec<KC> &x
 //   controller: `prepare` (wait for the dependency, build the activation vector in LDS; returns
 //               false to abandon), barrier, `overlap`, barrier, `finish` (epilogue + signal)
 // Both barriers are reached by all nine waves whatever the outcome of `prepare`.
-template <int KC, class RowOf, class Prepare, class Overlap, class Finish>
+template <int KC, int PF, class RowOf, class Prepare, class Overlap, class Finish>
 __device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need_x, RowOf row_ref, Prepare prepare,
                                              Overlap overlap, Finish finish) {
-    constexpr int PF = rows_in_flight<KC>();
     if (c.controller) {
         const bool ok = prepare();
         trace_event(c, kEvInputReady);
@@ -616,12 +631,16 @@ __device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need
     }
     const int mine = ntasks > c.wave ? (ntasks - c.wave + kConsumerWaves - 1) / kConsumerWaves : 0;
     uint4 buf[PF][KC];
-    // Every request below is issued unconditionally (rows past the end are no-op requests), so the
-    // count of outstanding loads at each wait is a compile-time constant: the wait for row i leaves
-    // the PF - 1 younger rows in flight.
+    // Requests are issued unconditionally wherever rows stream (rows past the end become no-op
+    // requests), so the count of outstanding loads at each wait is a compile-time constant: the
+    // wait for row i leaves the PF - 1 younger rows in flight.
     auto request = [&](uint4 (&dst)[KC], int i) {
         const bool valid = i < mine;
         load_row<KC>(dst, row_ref(valid ? c.wave + i * kConsumerWaves : 0), valid, c.lane);
+    };
+    auto consume = [&](const uint4 (&src)[KC], int i, const XVec<KC> &x) {
+        const float y = mkm::round_bf16(dot_row<KC>(src, x));
+        if (c.lane == 0) c.sm->out[c.wave + i * kConsumerWaves] = y;
     };
     trace_consumer(c, 20);
 #pragma unroll
@@ -632,19 +651,22 @@ __device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need
     XVec<KC> x;
     if (need_x) x_from_lds<KC>(x, c.sm, c.lane);
     trace_consumer(c, 24);
-    for (int base = 0; base < mine; base += PF) {
-        if (base == PF) trace_consumer(c, 25);
+    int base = 0;
+    // rounds that are followed by more rows: every row of the round exists, every slot is refilled
+    for (; base + PF < mine; base += PF) {
 #pragma unroll
         for (int s = 0; s < PF; s++) {
-            const int i = base + s;
-            float y = 0.0f;
-            if (i < mine) y = mkm::round_bf16(dot_row<KC>(buf[s], x));
+            consume(buf[s], base + s, x);
             compiler_fence();
-            request(buf[s], i + PF);
+            request(buf[s], base + s + PF);
             compiler_fence();
-            if (i < mine && c.lane == 0) c.sm->out[c.wave + i * kConsumerWaves] = y;
         }
     }
+    trace_consumer(c, 25);
+    // last round: nothing left to request
+#pragma unroll
+    for (int s = 0; s < PF; s++)
+        if (base + s < mine) consume(buf[s], base + s, x);
     trace_consumer(c, 23);
     wg_barrier();
     trace_consumer_flush(c, 20, 25);
@@ -682,7 +704,7 @@ static __device__ __noinline__ bool op_qkv(SmemPtr lds, int slot, int *refusal) 
     const WeightBuffer W = weight_buffer(a.qkv_weights + (size_t)layer * total_blocks * 16 * hid, matrix_bytes);
     const int down_jobs = (a.intermediate_size / a.matvec_reduction_size) * (hid / 16);
 
-    return matvec_batch<KC>(
+    return matvec_batch<KC, rows_in_flight<KC>(MK_PF_QKV)>(
         c, nblk * 16, nblk > 0, [&](int t) { return RowRef{W, (uint32_t)(start * 16 + t) * (uint32_t)hid * 2u}; },
         [&]() {
             uint4 wraw[KC];
@@ -736,8 +758,8 @@ static __device__ __noinline__ bool op_qkv(SmemPtr lds, int slot, int *refusal) 
 // residual in group order, which is the order the Python VM applies them in, so the bf16
 // rounding chain is reproduced without serialising the workers.
 // ---------------------------------------------------------------------------------------------
-template <int KC>
-static __device__ __noinline__ bool op_matvec_add(SmemPtr lds, int slot, bool is_down, int *refusal) {
+template <int KC, bool is_down>
+static __device__ __noinline__ bool op_matvec_add(SmemPtr lds, int slot, int *refusal) {
     const InsPtr ins = lds->queue[slot];
     const Ctx c = make_ctx(lds, slot, ins[0]);
     ArgsRef a = c.sm->args;
@@ -763,7 +785,7 @@ static __device__ __noinline__ bool op_matvec_add(SmemPtr lds, int slot, bool is
     uint32_t pre[kPre] = {0, 0};
     const bool prefetched = nblk * 8 <= kPre * 64;
 
-    return matvec_batch<KC>(
+    return matvec_batch<KC, rows_in_flight<KC>(is_down ? MK_PF_DOWN : MK_PF_OPROJ)>(
         c, nblk * 16, nblk > 0, [&](int t) { return RowRef{W, (uint32_t)(start * 16 + t) * (uint32_t)in_dim * 2u}; },
         [&]() {
             if (!poll_sharded(c, layer, wait_row, wait_target)) return false;
@@ -845,7 +867,7 @@ static __device__ __noinline__ bool op_upgate(SmemPtr lds, int slot, int *refusa
     const int o_jobs = (hid / a.matvec_reduction_size) * (hid / 16);
 
     // task t: list entry t / 32, matrix (t / 16) & 1 (0 up, 1 gate), row t % 16
-    return matvec_batch<KC>(
+    return matvec_batch<KC, rows_in_flight<KC>(MK_PF_UPGATE)>(
         c, n * 32, n > 0,
         [&](int t) {
             const int blk = ins[3 + (t >> 5)];
@@ -898,7 +920,7 @@ static __device__ __noinline__ bool op_lm_head(SmemPtr lds, int slot, int *refus
     do {
         const int b1 = min(b0 + blocks_per_batch, end);
         const int nblk = b1 > b0 ? b1 - b0 : 0;
-        const bool ok = matvec_batch<KC>(
+        const bool ok = matvec_batch<KC, rows_in_flight<KC>(MK_PF_LMHEAD)>(
             c, nblk * 16, true, [&](int t) { return RowRef{W, (uint32_t)(b0 * 16 + t) * (uint32_t)hid * 2u}; },
             [&]() {
                 if (!first) return true;  // the activation vector stays in LDS between batches
@@ -1371,9 +1393,9 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
         case 1: ok = op_qkv<KC_HID>(sm, slot, &refusal); break;
         case 2: ok = op_attention<D>(sm, slot, &refusal); break;
         case 3: ok = op_attention_reduction(sm, slot, &refusal); break;
-        case 4: ok = op_matvec_add<KC_RED>(sm, slot, false, &refusal); break;
+        case 4: ok = op_matvec_add<KC_RED, false>(sm, slot, &refusal); break;
         case 5: ok = op_upgate<KC_HID>(sm, slot, &refusal); break;
-        case 6: ok = op_matvec_add<KC_RED>(sm, slot, true, &refusal); break;
+        case 6: ok = op_matvec_add<KC_RED, true>(sm, slot, &refusal); break;
         case 7: ok = op_lm_head<KC_HID>(sm, slot, &refusal); break;
         default: ok = bail(make_ctx(sm, slot, opcode), MK_STATUS_BAD_OPCODE, &refusal);  // reference: trap, include/util.cuh:38
         }
