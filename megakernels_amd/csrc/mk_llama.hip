@@ -427,18 +427,31 @@ __device__ void record_status(const Ctx &c, int code) {
     }
 }
 
-// Executed by all lanes of the controller wave.  `ptr` is this lane's counter or nullptr.
+// First round of a dependency wait, requested ahead of time: the values this lane saw.
+struct PollTicket {
+    const int *ptr;
+    int value, status;
+};
+__device__ __forceinline__ PollTicket poll_issue(const Ctx &c, const int *ptr) {
+    PollTicket t;
+    t.ptr = ptr;
+    t.value = ptr ? ld_i32(ptr) : 0;
+    t.status = c.lane == 63 ? ld_i32(ws_status(c)) : 0;
+    return t;
+}
+
+// Executed by all lanes of the controller wave.  The ticket holds this lane's counter (or nullptr)
+// and the first values read from it.
 // sum_mode: wait until the sum over lanes reaches target (sharded counter + its base value);
 // otherwise wait until every lane's counter reaches target.  Lane 63 watches the global status
 // word so that one worker's failure releases everybody.
-__device__ bool poll_counters(const Ctx &c, const int *ptr, bool sum_mode, int target) {
+__device__ bool poll_wait(const Ctx &c, PollTicket t, bool sum_mode, int target) {
     const long long t0 = wall_clock64();
     const long long limit = spin_ticks(c);
     const int *status = ws_status(c);
+    int v = t.value, st = t.status;
     while (true) {
-        const int v = ptr ? ld_i32(ptr) : 0;
-        const int st = c.lane == 63 ? ld_i32(status) : 0;
-        const bool ok = sum_mode ? (lane_sum_i32(v) >= target) : (bool)__all(ptr == nullptr || v >= target);
+        const bool ok = sum_mode ? (lane_sum_i32(v) >= target) : (bool)__all(t.ptr == nullptr || v >= target);
         if (ok) break;
         if (__any(st != 0)) return false;
         if (wall_clock64() - t0 > limit) {
@@ -446,16 +459,23 @@ __device__ bool poll_counters(const Ctx &c, const int *ptr, bool sum_mode, int t
             return false;
         }
         __builtin_amdgcn_s_sleep(1);
+        v = t.ptr ? ld_i32(t.ptr) : 0;
+        st = c.lane == 63 ? ld_i32(status) : 0;
     }
     compiler_fence();  // data loads stay after the successful poll
     return true;
 }
+__device__ __forceinline__ bool poll_counters(const Ctx &c, const int *ptr, bool sum_mode, int target) {
+    return poll_wait(c, poll_issue(c, ptr), sum_mode, target);
+}
 
+__device__ __forceinline__ const int *sharded_lane_ptr(const Ctx &c, int layer, int row) {
+    if (c.lane < kShards) return shard_ptr(c, c.lane, layer, row);
+    if (c.lane == kShards) return bar_ptr(c, layer, row, 0);
+    return nullptr;
+}
 __device__ __forceinline__ bool poll_sharded(const Ctx &c, int layer, int row, int target) {
-    const int *p = nullptr;
-    if (c.lane < kShards) p = shard_ptr(c, c.lane, layer, row);
-    else if (c.lane == kShards) p = bar_ptr(c, layer, row, 0);
-    return poll_counters(c, p, true, target);
+    return poll_counters(c, sharded_lane_ptr(c, layer, row), true, target);
 }
 
 // one arrival on a sharded counter; the caller has waited for its stores
@@ -613,10 +633,18 @@ __device__ __forceinline__ float dot_row(const uint4 (&w)[KC], const XVec<KC> &x
 //   controller: `prepare` (wait for the dependency, build the activation vector in LDS; returns
 //               false to abandon), barrier, `overlap`, barrier, `finish` (epilogue + signal)
 // Both barriers are reached by all nine waves whatever the outcome of `prepare`.
-template <int KC, int PF, class RowOf, class Prepare, class Overlap, class Finish>
-__device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need_x, RowOf row_ref, Prepare prepare,
-                                             Overlap overlap, Finish finish) {
+template <int KC, int PF, class RowOf, class Ahead, class Prepare, class Overlap, class Finish>
+__device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need_x, RowOf row_ref, Ahead ahead,
+                                             Prepare prepare, Overlap overlap, Finish finish) {
     if (c.controller) {
+        // The controller's first requests: first look at the dependency, norm weights.  With
+        // MK_ENTRY_BARRIER they go out before the consumers' bulk requests (a CU serves its requests
+        // in order); measured, the activation load then queues behind the bulk instead and nothing
+        // is gained, so the barrier is off.
+        ahead();
+#ifdef MK_ENTRY_BARRIER
+        wg_barrier();
+#endif
         const bool ok = prepare();
         trace_event(c, kEvInputReady);
         if (!barrier_inputs_ready(c, ok)) return false;
@@ -642,6 +670,9 @@ __device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need
         const float y = mkm::round_bf16(dot_row<KC>(src, x));
         if (c.lane == 0) c.sm->out[c.wave + i * kConsumerWaves] = y;
     };
+#ifdef MK_ENTRY_BARRIER
+    wg_barrier();
+#endif
     trace_consumer(c, 20);
 #pragma unroll
     for (int s = 0; s < PF; s++) request(buf[s], s);
@@ -703,13 +734,17 @@ static __device__ __noinline__ bool op_qkv(SmemPtr lds, int slot, int *refusal) 
     const size_t matrix_bytes = (size_t)total_blocks * 16 * hid * 2;
     const WeightBuffer W = weight_buffer(a.qkv_weights + (size_t)layer * total_blocks * 16 * hid, matrix_bytes);
     const int down_jobs = (a.intermediate_size / a.matvec_reduction_size) * (hid / 16);
+    PollTicket ticket = {nullptr, 0, 0};
+    uint4 wraw[KC];
 
     return matvec_batch<KC, rows_in_flight<KC>(MK_PF_QKV)>(
         c, nblk * 16, nblk > 0, [&](int t) { return RowRef{W, (uint32_t)(start * 16 + t) * (uint32_t)hid * 2u}; },
         [&]() {
-            uint4 wraw[KC];
+            if (layer > 0) ticket = poll_issue(c, sharded_lane_ptr(c, layer - 1, 5));
             if (nblk > 0) load_row<KC>(wraw, a.attn_norm_weights + (size_t)layer * hid, c.lane);
-            if (layer > 0 && !poll_sharded(c, layer - 1, 5, down_jobs)) return false;
+        },
+        [&]() {
+            if (layer > 0 && !poll_wait(c, ticket, true, down_jobs)) return false;
             trace_event(c, kEvDepReady);
             if (nblk > 0) {
                 uint4 xq[KC];
@@ -784,11 +819,13 @@ static __device__ __noinline__ bool op_matvec_add(SmemPtr lds, int slot, int *re
     constexpr int kPre = 2;
     uint32_t pre[kPre] = {0, 0};
     const bool prefetched = nblk * 8 <= kPre * 64;
+    PollTicket ticket = {nullptr, 0, 0};
 
     return matvec_batch<KC, rows_in_flight<KC>(is_down ? MK_PF_DOWN : MK_PF_OPROJ)>(
         c, nblk * 16, nblk > 0, [&](int t) { return RowRef{W, (uint32_t)(start * 16 + t) * (uint32_t)in_dim * 2u}; },
+        [&]() { ticket = poll_issue(c, sharded_lane_ptr(c, layer, wait_row)); },
         [&]() {
-            if (!poll_sharded(c, layer, wait_row, wait_target)) return false;
+            if (!poll_wait(c, ticket, true, wait_target)) return false;
             trace_event(c, kEvDepReady);
             if (nblk > 0) {
                 uint4 xq[KC];
@@ -865,6 +902,8 @@ static __device__ __noinline__ bool op_upgate(SmemPtr lds, int slot, int *refusa
     const WeightBuffer Wu = weight_buffer(a.up_weights + (size_t)layer * inter * hid, matrix_bytes);
     const WeightBuffer Wg = weight_buffer(a.gate_weights + (size_t)layer * inter * hid, matrix_bytes);
     const int o_jobs = (hid / a.matvec_reduction_size) * (hid / 16);
+    PollTicket ticket = {nullptr, 0, 0};
+    uint4 wraw[KC];
 
     // task t: list entry t / 32, matrix (t / 16) & 1 (0 up, 1 gate), row t % 16
     return matvec_batch<KC, rows_in_flight<KC>(MK_PF_UPGATE)>(
@@ -874,9 +913,11 @@ static __device__ __noinline__ bool op_upgate(SmemPtr lds, int slot, int *refusa
             return RowRef{(t >> 4) & 1 ? Wg : Wu, (uint32_t)(blk * 16 + (t & 15)) * (uint32_t)hid * 2u};
         },
         [&]() {
-            uint4 wraw[KC];
+            ticket = poll_issue(c, sharded_lane_ptr(c, layer, 3));
             if (n > 0) load_row<KC>(wraw, a.mlp_norm_weights + (size_t)layer * hid, c.lane);
-            if (!poll_sharded(c, layer, 3, o_jobs)) return false;
+        },
+        [&]() {
+            if (!poll_wait(c, ticket, true, o_jobs)) return false;
             trace_event(c, kEvDepReady);
             if (n > 0) {
                 uint4 xq[KC];
@@ -915,6 +956,8 @@ static __device__ __noinline__ bool op_lm_head(SmemPtr lds, int slot, int *refus
     const int down_jobs = (a.intermediate_size / a.matvec_reduction_size) * (hid / 16);
     const int blocks_per_batch = kOutRows / 16;
     const WeightBuffer W = weight_buffer(a.lm_head_weights, (size_t)a.vocab_size * hid * 2);
+    PollTicket ticket = {nullptr, 0, 0};
+    uint4 wraw[KC];
     bool first = true;
     int b0 = start;
     do {
@@ -923,10 +966,13 @@ static __device__ __noinline__ bool op_lm_head(SmemPtr lds, int slot, int *refus
         const bool ok = matvec_batch<KC, rows_in_flight<KC>(MK_PF_LMHEAD)>(
             c, nblk * 16, true, [&](int t) { return RowRef{W, (uint32_t)(b0 * 16 + t) * (uint32_t)hid * 2u}; },
             [&]() {
-                if (!first) return true;  // the activation vector stays in LDS between batches
-                uint4 wraw[KC];
+                if (!first) return;
+                ticket = poll_issue(c, sharded_lane_ptr(c, a.num_layers - 1, 5));
                 load_row<KC>(wraw, a.lm_head_norm_weights, c.lane);
-                if (!poll_sharded(c, a.num_layers - 1, 5, down_jobs)) return false;
+            },
+            [&]() {
+                if (!first) return true;  // the activation vector stays in LDS between batches
+                if (!poll_wait(c, ticket, true, down_jobs)) return false;
                 trace_event(c, kEvDepReady);
                 uint4 xq[KC];
                 rms_norm_x<KC>(xq, a.hidden_states, wraw, a.rms_norm_eps, c.lane);
