@@ -48,7 +48,6 @@ namespace {
 constexpr int kConsumerWaves = 8;
 constexpr int kConsumerThreads = kConsumerWaves * 64;
 constexpr int kThreads = kConsumerThreads + 64;  // + one controller wave
-constexpr int kVirtualWaves = 16;   // attention slot layout is defined for 16 waves; each consumer wave plays two
 #ifndef MK_SHARDS
 #define MK_SHARDS 16
 #endif
@@ -126,16 +125,20 @@ struct Smem {
 #ifdef MK_TRACE_CONSUMER
     int consumer_ticks[16];         // development trace: consumer timestamps parked until the instruction ends
 #endif
-    uint32_t x[kMaxK / 2];          // activation vector as bf16 pairs, lane layout [chunk][lane][4 dwords]
-    float out[kOutRows];            // matvec row results awaiting the epilogue
-    float wave_max[kVirtualWaves][kGqa];
-    float wave_l[kVirtualWaves][kGqa];
+    alignas(16) uint32_t x[kMaxK / 2];          // activation vector as bf16 pairs, lane layout [chunk][lane][4 dwords]
+    alignas(16) float out[kOutRows];            // matvec row results awaiting the epilogue
+    alignas(16) float wave_max[kConsumerWaves][kGqa];
+    alignas(16) float wave_l[kConsumerWaves][kGqa];
     float head_m[kGqa];
     float head_w[kGqa][32];         // reduction weights
-    float wave_o[kVirtualWaves][kGqa][kMaxHeadDim];
-    float scores[kGqa][kScoreCap];
+    alignas(16) float wave_o[kConsumerWaves][kGqa][kMaxHeadDim];
+    alignas(16) float scores[kScoreCap][kGqa];  // attention: one partition's scores, then probabilities
     int queue[kQueueSlots][MK_INSTRUCTION_WORDS];  // this worker's instructions, fetched once
 };
+static_assert(offsetof(Smem, x) % 16 == 0 && offsetof(Smem, wave_max) % 16 == 0 && offsetof(Smem, wave_l) % 16 == 0 &&
+                  offsetof(Smem, scores) % 16 == 0,
+              "128-bit LDS accesses need 16-byte aligned members");
+
 static_assert(sizeof(Smem) <= 160 * 1024, "LDS budget");
 static_assert(sizeof(Smem) > 80 * 1024, "must keep a second workgroup off the CU");
 
@@ -479,8 +482,11 @@ __device__ __forceinline__ bool poll_sharded(const Ctx &c, int layer, int row, i
 }
 
 // one arrival on a sharded counter; the caller has waited for its stores
+__device__ __forceinline__ void signal_sharded_lane(const Ctx &c, int layer, int row, int count) {
+    add_i32(shard_ptr(c, c.worker & (kShards - 1), layer, row), count);
+}
 __device__ __forceinline__ void signal_sharded(const Ctx &c, int layer, int row, int count) {
-    if (c.lane == 0) add_i32(shard_ptr(c, c.worker & (kShards - 1), layer, row), count);
+    if (c.lane == 0) signal_sharded_lane(c, layer, row, count);
 }
 
 // Controller: publish the outcome of the dependency wait; everybody: first barrier of the
@@ -1014,19 +1020,18 @@ __device__ __forceinline__ void halving_level(float *vals, int lane) {
 // (python_vm.py:277-346; reference device op: demos/low-latency-llama/attention_partial.cu).
 // Two passes over LDS-resident scores: (1) s = scale * q.k for every token, exact maximum;
 // (2) p = exp(s - max), slot sums of p and p*v.  Token r of the partition belongs to slot
-// r mod NSLOT, NSLOT = 16 virtual waves * (64 / (D/8)) tokens per wave load; a slot accumulates
-// its tokens in increasing order and slots are combined by a pairwise tree (lanes, then virtual
-// waves).  Each of the 8 consumer waves plays virtual waves w and w + 8.
+// r mod NSLOT, NSLOT = 8 waves * (64 / (D/8)) tokens per wave load; a slot accumulates its
+// tokens in increasing order and slots are combined by a pairwise tree (token groups of a wave,
+// then waves).  A token's row is spread over D/8 lanes, 8 dims each.
 // ---------------------------------------------------------------------------------------------
 template <int D>
 static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *refusal) {
     const InsPtr ins = lds->queue[slot];
     const Ctx c = make_ctx(lds, slot, ins[0]);
-    constexpr int LPT = D / 8;                  // lanes per token
-    constexpr int TPW = 64 / LPT;               // tokens per wave per round
-    constexpr int NSLOT = kVirtualWaves * TPW;  // tokens per workgroup round
+    constexpr int LPT = D / 8;                   // lanes per token
+    constexpr int TPW = 64 / LPT;                // tokens per wave per round
+    constexpr int NSLOT = kConsumerWaves * TPW;  // tokens per workgroup round
     constexpr int G = kGqa;
-    constexpr int VW = kVirtualWaves / kConsumerWaves;  // virtual waves per consumer wave
     ArgsRef a = c.sm->args;
     const SmemPtr sm = c.sm;
     const int layer = ins[1], kvh = ins[2], P = ins[3], pidx = ins[4];
@@ -1062,10 +1067,8 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
         trace_event(c, 7);
         wg_barrier();  // wave sums
         trace_event(c, 8);
-        wg_barrier();  // outputs stored
         trace_event(c, kEvComputeDone);
-        if (skip) signal_sharded(c, layer, 2, G);
-        else if (c.lane < G) add_i32(bar_ptr(c, layer, 1, h0 + c.lane), 1);
+        // the waves that combine the sums store and signal on their own
         return true;
     }
 
@@ -1075,8 +1078,8 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
     const size_t base = ((size_t)layer * a.kv_max_len) * tok_stride + (size_t)kvh * D + sub * 8;
     const uint16_t *kbase = a.k_cache + base;
     const uint16_t *vbase = a.v_cache + base;
-    // relative token handled by this lane in round rd as virtual wave v
-    auto token_of = [&](int rd, int v) { return rd * NSLOT + (c.wave + v * kConsumerWaves) * TPW + tok_in_wave; };
+    // relative token handled by this lane in round rd
+    auto token_of = [&](int rd) { return rd * NSLOT + c.wave * TPW + tok_in_wave; };
     // rows older than this step are immutable; the row at pos_id was written by another CU a moment
     // ago and needs a coherent load
     auto load_kv = [&](const uint16_t *kvb, int r) {
@@ -1085,19 +1088,20 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
         return t == a.pos_id ? ld_b128(p) : ld_const_b128(p);
     };
 
-    // Rounds are processed in batches of RU so that RU * VW row loads are in flight per lane.  The
-    // first batch of K does not depend on this step except for the newest token: request it before
+    // Rounds are processed in batches of RU so that RU row loads are in flight per lane.  The first
+    // batch of K and V does not depend on this step except for the newest token: request it before
     // the dependency is known.
-    constexpr int RU = 2;
-    uint4 kraw[RU][VW], vraw[RU][VW];
+    constexpr int RU = 4;
+    uint4 kraw[RU], vraw[RU];
 #pragma unroll
-    for (int u = 0; u < RU; u++)
-#pragma unroll
-        for (int v = 0; v < VW; v++) {
-            const int r = token_of(u, v);
-            kraw[u][v] = make_uint4(0, 0, 0, 0);
-            if (r < T && t0 + r != a.pos_id) kraw[u][v] = ld_const_b128(kbase + (size_t)(t0 + r) * tok_stride);
+    for (int u = 0; u < RU; u++) {
+        const int r = token_of(u);
+        kraw[u] = vraw[u] = make_uint4(0, 0, 0, 0);
+        if (r < T && t0 + r != a.pos_id) {
+            kraw[u] = ld_const_b128(kbase + (size_t)(t0 + r) * tok_stride);
+            vraw[u] = ld_const_b128(vbase + (size_t)(t0 + r) * tok_stride);
         }
+    }
     if (!barrier_inputs_ready(c, true)) return false;
     trace_consumer(c, 16);
 
@@ -1106,179 +1110,162 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
         uint4 qraw[G];
 #pragma unroll
         for (int h = 0; h < G; h++) qraw[h] = ld_b128(a.q_post_rope + (size_t)(h0 + h) * D + sub * 8);
-        // the newest token's K row, if it falls into the first batch
+        // the newest token's rows, if they fall into the first batch
 #pragma unroll
-        for (int u = 0; u < RU; u++)
-#pragma unroll
-            for (int v = 0; v < VW; v++) {
-                const int r = token_of(u, v);
-                if (r < T && t0 + r == a.pos_id) kraw[u][v] = ld_b128(kbase + (size_t)(t0 + r) * tok_stride);
+        for (int u = 0; u < RU; u++) {
+            const int r = token_of(u);
+            if (r < T && t0 + r == a.pos_id) {
+                kraw[u] = ld_b128(kbase + (size_t)(t0 + r) * tok_stride);
+                vraw[u] = ld_b128(vbase + (size_t)(t0 + r) * tok_stride);
             }
+        }
 #pragma unroll
         for (int h = 0; h < G; h++) unpack8(qraw[h], q[h]);
     }
-    if (q[0][0] == 12345.0f) trace_consumer(c, 31);  // forces the loads to have landed
     trace_consumer(c, 17);
 
-    // ---- pass 1: scores and maximum ----
-    float mx[VW][G];
+    // ---- pass 1: scores (kept as [token][head] in LDS) and maximum ----
+    float mx[G];
 #pragma unroll
-    for (int v = 0; v < VW; v++)
-#pragma unroll
-        for (int h = 0; h < G; h++) mx[v][h] = -INFINITY;
+    for (int h = 0; h < G; h++) mx[h] = -INFINITY;
     for (int rb = 0; rb < rounds; rb += RU) {
         if (rb > 0) {
 #pragma unroll
-            for (int u = 0; u < RU; u++)
-#pragma unroll
-                for (int v = 0; v < VW; v++) {
-                    const int r = token_of(rb + u, v);
-                    if (r < T) kraw[u][v] = load_kv(kbase, r);
-                }
-        } else {
-            // the first batch of V can be requested now: it is needed right after the maximum
-#pragma unroll
-            for (int u = 0; u < RU; u++)
-#pragma unroll
-                for (int v = 0; v < VW; v++) {
-                    const int r = token_of(u, v);
-                    vraw[u][v] = make_uint4(0, 0, 0, 0);
-                    if (r < T) vraw[u][v] = load_kv(vbase, r);
-                }
+            for (int u = 0; u < RU; u++) {
+                const int r = token_of(rb + u);
+                if (r < T) kraw[u] = load_kv(kbase, r);
+            }
         }
 #pragma unroll
-        for (int u = 0; u < RU; u++)
+        for (int u = 0; u < RU; u++) {
+            const int r = token_of(rb + u);
+            if (r < T) {  // the LPT lanes of a token share r, so they are active together
+                float kf[8], sc[G];
+                unpack8(kraw[u], kf);
 #pragma unroll
-            for (int v = 0; v < VW; v++) {
-                const int r = token_of(rb + u, v);
-                if (r < T) {  // the LPT lanes of a token share r, so they are active together
-                    float kf[8];
-                    unpack8(kraw[u][v], kf);
+                for (int h = 0; h < G; h++) {
+                    float acc = 0.0f;
 #pragma unroll
-                    for (int h = 0; h < G; h++) {
-                        float acc = 0.0f;
-#pragma unroll
-                        for (int e = 0; e < 8; e++) acc = fmaf(q[h][e], kf[e], acc);
-                        const float s = group_tree_sum<LPT>(acc) * a.attn_scale;
-                        if (sub == 0) sm->scores[h][r] = s;
-                        mx[v][h] = fmaxf(mx[v][h], s);
-                    }
+                    for (int e = 0; e < 8; e++) acc = fmaf(q[h][e], kf[e], acc);
+                    sc[h] = group_tree_sum<LPT>(acc) * a.attn_scale;
+                    mx[h] = fmaxf(mx[h], sc[h]);
                 }
+                if (sub == 0) *(MK_LDS f32x4 *)&sm->scores[r][0] = f32x4{sc[0], sc[1], sc[2], sc[3]};
             }
+        }
     }
     trace_consumer(c, 18);
+    {
+        float m[G];
 #pragma unroll
-    for (int v = 0; v < VW; v++)
-#pragma unroll
-        for (int h = 0; h < G; h++) {
-            const float m = lane_tree_max<LPT, 64>(mx[v][h]);
-            if (c.lane == 0) sm->wave_max[c.wave + v * kConsumerWaves][h] = m;
-        }
+        for (int h = 0; h < G; h++) m[h] = lane_tree_max<LPT, 64>(mx[h]);
+        if (c.lane == 0) *(MK_LDS f32x4 *)&sm->wave_max[c.wave][0] = f32x4{m[0], m[1], m[2], m[3]};
+    }
     trace_consumer(c, 19);
     wg_barrier();
     trace_consumer_flush(c, 16, 19);
     float hm[G];
+    {
+        f32x4 m = *(const MK_LDS f32x4 *)&sm->wave_max[0][0];
 #pragma unroll
-    for (int h = 0; h < G; h++) {
-        float m = sm->wave_max[0][h];
-        for (int w = 1; w < kVirtualWaves; w++) m = fmaxf(m, sm->wave_max[w][h]);
-        hm[h] = m;
+        for (int w = 1; w < kConsumerWaves; w++) {
+            const f32x4 o = *(const MK_LDS f32x4 *)&sm->wave_max[w][0];
+            m.x = fmaxf(m.x, o.x); m.y = fmaxf(m.y, o.y); m.z = fmaxf(m.z, o.z); m.w = fmaxf(m.w, o.w);
+        }
+        hm[0] = m.x; hm[1] = m.y; hm[2] = m.z; hm[3] = m.w;
     }
-    // p = exp(s - max), once per (head, token), in place
-    for (int i = c.tid; i < G * T; i += kConsumerThreads) {
-        const int h = i / T, r = i - h * T;
-        const float m = h == 0 ? hm[0] : h == 1 ? hm[1] : h == 2 ? hm[2] : hm[3];
-        sm->scores[h][r] = mkm::expf_exact(sm->scores[h][r] - m);
+    // p = exp(s - max), once per (token, head), in place
+    {
+        MK_LDS float *flat = &sm->scores[0][0];
+        for (int i = c.tid; i < G * T; i += kConsumerThreads) {
+            const int h = i & (G - 1);
+            const float m = h == 0 ? hm[0] : h == 1 ? hm[1] : h == 2 ? hm[2] : hm[3];
+            flat[i] = mkm::expf_exact(flat[i] - m);
+        }
     }
     wg_barrier();
 
     // ---- pass 2: slot sums ----
-    float acc[VW][G][8], lsum[VW][G];
+    float acc[G][8], lsum[G];
 #pragma unroll
-    for (int v = 0; v < VW; v++)
+    for (int h = 0; h < G; h++) {
+        lsum[h] = 0.0f;
 #pragma unroll
-        for (int h = 0; h < G; h++) {
-            lsum[v][h] = 0.0f;
-#pragma unroll
-            for (int e = 0; e < 8; e++) acc[v][h][e] = 0.0f;
-        }
+        for (int e = 0; e < 8; e++) acc[h][e] = 0.0f;
+    }
     for (int rb = 0; rb < rounds; rb += RU) {
         if (rb > 0) {
 #pragma unroll
-            for (int u = 0; u < RU; u++)
-#pragma unroll
-                for (int v = 0; v < VW; v++) {
-                    const int r = token_of(rb + u, v);
-                    if (r < T) vraw[u][v] = load_kv(vbase, r);
-                }
+            for (int u = 0; u < RU; u++) {
+                const int r = token_of(rb + u);
+                if (r < T) vraw[u] = load_kv(vbase, r);
+            }
         }
 #pragma unroll
-        for (int u = 0; u < RU; u++)
+        for (int u = 0; u < RU; u++) {
+            const int r = token_of(rb + u);
+            if (r < T) {
+                float vf[8];
+                unpack8(vraw[u], vf);
+                const f32x4 pv = *(const MK_LDS f32x4 *)&sm->scores[r][0];
+                const float p[G] = {pv.x, pv.y, pv.z, pv.w};
 #pragma unroll
-            for (int v = 0; v < VW; v++) {
-                const int r = token_of(rb + u, v);
-                if (r < T) {
-                    float vf[8];
-                    unpack8(vraw[u][v], vf);
+                for (int h = 0; h < G; h++) {
+                    lsum[h] = lsum[h] + p[h];
 #pragma unroll
-                    for (int h = 0; h < G; h++) {
-                        const float p = sm->scores[h][r];
-                        lsum[v][h] = lsum[v][h] + p;
-#pragma unroll
-                        for (int e = 0; e < 8; e++) acc[v][h][e] = fmaf(p, vf[e], acc[v][h][e]);
-                    }
+                    for (int e = 0; e < 8; e++) acc[h][e] = fmaf(p[h], vf[e], acc[h][e]);
                 }
             }
+        }
     }
-    // Combine the TPW slots of each virtual wave: a pairwise tree over the token groups (lane bits
+    // Combine the TPW slots of the wave: a pairwise tree over the token groups (lane bits
     // log2(LPT) .. 5).  Recursive halving: at each level a lane hands half of its partial sums to
     // its partner and keeps the other half, so the 32 sums per lane shrink to 32 / TPW and the
     // number of lane exchanges drops from 32 per level to 16 + 8 + 4.  own + partner is the same
     // addition the butterfly would do.
-#pragma unroll
-    for (int v = 0; v < VW; v++) {
+    {
         float part[G * 8];
 #pragma unroll
         for (int h = 0; h < G; h++)
 #pragma unroll
-            for (int e = 0; e < 8; e++) part[h * 8 + e] = acc[v][h][e];
+            for (int e = 0; e < 8; e++) part[h * 8 + e] = acc[h][e];
         halving_level<LPT, G * 8>(part, c.lane);
         halving_level<LPT * 2, G * 4>(part, c.lane);
         if constexpr (TPW == 8) halving_level<LPT * 4, G * 2>(part, c.lane);
         // the lane now holds the sums with index  tg_bit0 * 16 + tg_bit1 * 8 (+ tg_bit2 * 4) + k
         constexpr int kLeft = G * 8 / TPW;
         const int first = ((tok_in_wave & 1) * 16) + (((tok_in_wave >> 1) & 1) * 8) + (TPW == 8 ? ((tok_in_wave >> 2) & 1) * 4 : 0);
-        MK_LDS float *dst = &sm->wave_o[c.wave + v * kConsumerWaves][0][0];
+        MK_LDS float *dst = &sm->wave_o[c.wave][0][0];
 #pragma unroll
         for (int k = 0; k < kLeft; k++) {
             const int idx = first + k;  // = h * 8 + e
             dst[(idx >> 3) * kMaxHeadDim + sub * 8 + (idx & 7)] = part[k];
         }
+        float l[G];
 #pragma unroll
-        for (int h = 0; h < G; h++) {
-            const float l = lane_tree_sum<LPT, 64>(lsum[v][h]);
-            if (c.lane == 0) sm->wave_l[c.wave + v * kConsumerWaves][h] = l;
-        }
+        for (int h = 0; h < G; h++) l[h] = lane_tree_sum<LPT, 64>(lsum[h]);
+        if (c.lane == 0) *(MK_LDS f32x4 *)&sm->wave_l[c.wave][0] = f32x4{l[0], l[1], l[2], l[3]};
     }
     wg_barrier();
 
-    // ---- combine the 16 virtual waves pairwise, normalise, store: thread -> (head, dim pair) ----
+    // ---- combine the 8 waves pairwise, normalise, store: thread -> (head, dim pair).  The threads of
+    // one head sit in one wave, which signals for that head once its own stores have landed. ----
     if (c.tid < G * D / 2) {
         const int h = c.tid / (D / 2), d = (c.tid % (D / 2)) * 2;
-        float o0[kVirtualWaves], o1[kVirtualWaves], l[kVirtualWaves];
+        float o0[kConsumerWaves], o1[kConsumerWaves], l[kConsumerWaves];
 #pragma unroll
-        for (int w = 0; w < kVirtualWaves; w++) {
+        for (int w = 0; w < kConsumerWaves; w++) {
             o0[w] = sm->wave_o[w][h][d];
             o1[w] = sm->wave_o[w][h][d + 1];
             l[w] = sm->wave_l[w][h];
         }
 #pragma unroll
-        for (int s = 1; s < kVirtualWaves; s <<= 1)
+        for (int st = 1; st < kConsumerWaves; st <<= 1)
 #pragma unroll
-            for (int i = 0; i < kVirtualWaves; i += 2 * s) {
-                o0[i] = o0[i] + o0[i + s];
-                o1[i] = o1[i] + o1[i + s];
-                l[i] = l[i] + l[i + s];
+            for (int i = 0; i < kConsumerWaves; i += 2 * st) {
+                o0[i] = o0[i] + o0[i + st];
+                o1[i] = o1[i] + o1[i + st];
+                l[i] = l[i] + l[i + st];
             }
         const int head = h0 + h;
         float r0, r1, lse;
@@ -1299,9 +1286,12 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
             st_f32(dst + 1, r1);
             if (d == 0) st_f32(a.attn_lse_intermediates + (size_t)head * a.max_partials + pidx, lse);
         }
+        wait_stores();
+        if (d == 0) {
+            if (skip) signal_sharded_lane(c, layer, 2, 1);
+            else add_i32(bar_ptr(c, layer, 1, head), 1);
+        }
     }
-    wait_stores();
-    wg_barrier();
     return true;
 }
 

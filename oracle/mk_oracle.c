@@ -36,7 +36,7 @@
  *   l*8 .. l*8+7 in order with fused multiply-add and the lanes are added as a
  *   balanced binary tree.
  *   Attention over a token range: relative token r goes to slot r mod NSLOT
- *   (NSLOT = 8192/D); each slot accumulates its tokens in increasing order
+ *   (NSLOT = 4096/D); each slot accumulates its tokens in increasing order
  *   (fused multiply-add for p*v, plain add for the denominator); the slots
  *   are combined by the same pairwise tree.  The softmax maximum is exact in
  *   any order.  exp / exp2 / log2 are the polynomial kernels of exact_math.h.
@@ -218,7 +218,7 @@ static int op_partial_attention(mk_oracle_globals *g, const int32_t *w) {
     const int T = t1 > t0 ? t1 - t0 : 0;
 
     const int LPT = D / 8;            /* lanes per token */
-    const int NSLOT = 16 * (64 / LPT);
+    const int NSLOT = 8 * (64 / LPT);
     const size_t tok_stride = (size_t)KVH * D;
     const uint16_t *kbase = g->k_cache + ((size_t)layer * g->kv_max_len) * tok_stride + (size_t)kvh * D;
     const uint16_t *vbase = g->v_cache + ((size_t)layer * g->kv_max_len) * tok_stride + (size_t)kvh * D;
