@@ -129,8 +129,6 @@ struct Smem {
     alignas(16) float out[kOutRows];            // matvec row results awaiting the epilogue
     alignas(16) float wave_max[kConsumerWaves][kGqa];
     alignas(16) float wave_l[kConsumerWaves][kGqa];
-    float head_m[kGqa];
-    float head_w[kGqa][32];         // reduction weights
     alignas(16) float wave_o[kConsumerWaves][kGqa][kMaxHeadDim];
     alignas(16) float scores[kScoreCap][kGqa];  // attention: one partition's scores, then probabilities
     int queue[kQueueSlots][MK_INSTRUCTION_WORDS];  // this worker's instructions, fetched once
@@ -1251,6 +1249,7 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
     // ---- combine the 8 waves pairwise, normalise, store: thread -> (head, dim pair).  The threads of
     // one head sit in one wave, which signals for that head once its own stores have landed. ----
     if (c.tid < G * D / 2) {
+        trace_consumer(c, 29);
         const int h = c.tid / (D / 2), d = (c.tid % (D / 2)) * 2;
         float o0[kConsumerWaves], o1[kConsumerWaves], l[kConsumerWaves];
 #pragma unroll
@@ -1286,11 +1285,14 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
             st_f32(dst + 1, r1);
             if (d == 0) st_f32(a.attn_lse_intermediates + (size_t)head * a.max_partials + pidx, lse);
         }
+        trace_consumer(c, 30);
         wait_stores();
+        trace_consumer(c, 31);
         if (d == 0) {
             if (skip) signal_sharded_lane(c, layer, 2, 1);
             else add_i32(bar_ptr(c, layer, 1, head), 1);
         }
+        trace_consumer_flush(c, 29, 31);
     }
     return true;
 }
@@ -1299,15 +1301,19 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
 // opcode 3: log-sum-exp merge of attention partitions  (python_vm.py:349-393;
 // reference device op: demos/low-latency-llama/attention_reduction.cu:18-339)
 // ---------------------------------------------------------------------------------------------
+template <int D>
 static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot, int *refusal) {
     const InsPtr ins = lds->queue[slot];
     const Ctx c = make_ctx(lds, slot, ins[0]);
     ArgsRef a = c.sm->args;
     const SmemPtr sm = c.sm;
+    constexpr int kMaxList = MK_INSTRUCTION_WORDS - 7;
+    constexpr int TPH = D / 2;  // threads per head, two output dims each; all in one wave
+    static_assert(TPH >= kMaxList && TPH <= 64, "a head's threads also fetch one list entry's log-sum-exp each");
     const int layer = ins[1], hs = ins[2], P = ins[3], terminal = ins[4], n = ins[5];
-    const int D = a.head_dim, R = a.attn_reduction_size, MP = a.max_partials;
-    bool bad = layer < 0 || layer >= a.num_layers || n < 1 || n > MK_INSTRUCTION_WORDS - 7 || hs < 0 ||
-               hs + R > a.num_attention_heads || R > kGqa;
+    const int R = a.attn_reduction_size, MP = a.max_partials;
+    bool bad = layer < 0 || layer >= a.num_layers || n < 1 || n > kMaxList || hs < 0 ||
+               hs + R > a.num_attention_heads || R > kGqa || a.head_dim != D;
     if (!bad)
         for (int i = 0; i < n; i++) bad |= ins[6 + i] < 0 || ins[6 + i] >= MP;
     const int out_idx = bad ? 0 : ins[6 + n];
@@ -1318,50 +1324,46 @@ static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot
         const int *p = c.lane < R ? bar_ptr(c, layer, 1, hs + c.lane) : nullptr;
         const bool ok = poll_counters(c, p, false, P);
         trace_event(c, kEvDepReady);
-        if (ok) {
-            // weights 2^(lse_i - max) once per (head, list entry): lane i takes list entry i, so the
-            // loads of one head go out together
-            float lse[kGqa];
-#pragma unroll
-            for (int h = 0; h < kGqa; h++) {
-                const float *lses = a.attn_lse_intermediates + (size_t)(hs + h) * MP;
-                lse[h] = (h < R && c.lane < n) ? ld_f32(lses + ins[6 + c.lane]) : -INFINITY;
-            }
-#pragma unroll
-            for (int h = 0; h < kGqa; h++) {
-                const float m = lane_tree_max(lse[h]);
-                if (h < R && c.lane < n) sm->head_w[h][c.lane] = mkm::exp2f_exact(lse[h] - m);
-                if (h < R && c.lane == 0) sm->head_m[h] = m;
-            }
-        }
         if (!barrier_inputs_ready(c, ok)) return false;
-        wg_barrier();  // outputs stored
         trace_event(c, kEvComputeDone);
-        signal_sharded(c, layer, 2, R);
+        // the waves that merge the partitions store and signal on their own
         return true;
     }
     if (!barrier_inputs_ready(c, true)) return false;
-    if (c.tid < R * D / 2) {
-        const int h = c.tid / (D / 2), d = (c.tid % (D / 2)) * 2;
+    if (c.tid < R * TPH) {
+        const int h = c.tid / TPH, j = c.tid % TPH, d = j * 2;
         const int head = hs + h;
         const float *outs = a.attn_out_intermediates + (size_t)head * MP * D;
+        const float *lses = a.attn_lse_intermediates + (size_t)head * MP;
+        // every request goes out at once: this thread's two dims of each listed partition, and the
+        // log-sum-exp of list entry j
+        const float lse = j < n ? ld_f32(lses + ins[6 + j]) : -INFINITY;
+        uint64_t v[kMaxList];
+#pragma unroll
+        for (int k = 0; k < kMaxList; k++)
+            if (k < n) v[k] = ld_u64(outs + (size_t)ins[6 + k] * D + d);
+        // weights 2^(lse_i - max): lane j of the head's lane group holds the weight of list entry j
+        const float m = lane_tree_max<1, TPH>(lse);
+        const float wj = j < n ? mkm::exp2f_exact(lse - m) : 0.0f;
+        trace_consumer(c, 26);
         float den = 0.0f, o0 = 0.0f, o1 = 0.0f;
-        // accumulate in list order; the loads of up to 13 entries are issued together
-        constexpr int kBatch = 13;
-        for (int i0 = 0; i0 < n; i0 += kBatch) {
-            uint64_t v[kBatch];
+        // accumulate in list order; entry k's weight comes from lane k of this head's group
 #pragma unroll
-            for (int k = 0; k < kBatch; k++)
-                if (i0 + k < n) v[k] = ld_u64(outs + (size_t)ins[6 + i0 + k] * D + d);
-#pragma unroll
-            for (int k = 0; k < kBatch; k++)
-                if (i0 + k < n) {
-                    const float w = sm->head_w[h][i0 + k];
-                    den = den + w;
-                    o0 = fmaf(w, mkm::bits_f32((uint32_t)v[k]), o0);
-                    o1 = fmaf(w, mkm::bits_f32((uint32_t)(v[k] >> 32)), o1);
+        for (int k = 0; k < kMaxList; k++)
+            if (k < n) {
+                float w;
+                if constexpr (TPH == 64) {
+                    w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), k));
+                } else {
+                    const float w_lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), k));
+                    const float w_hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), k + 32));
+                    w = c.lane < 32 ? w_lo : w_hi;
                 }
-        }
+                den = den + w;
+                o0 = fmaf(w, mkm::bits_f32((uint32_t)v[k]), o0);
+                o1 = fmaf(w, mkm::bits_f32((uint32_t)(v[k] >> 32)), o1);
+            }
+        trace_consumer(c, 27);
         o0 = o0 / den;
         o1 = o1 / den;
         if (terminal) {
@@ -1370,12 +1372,13 @@ static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot
             float *dst = a.attn_out_intermediates + ((size_t)head * MP + out_idx) * D + d;
             st_f32(dst, o0);
             st_f32(dst + 1, o1);
-            if (d == 0)
-                st_f32(a.attn_lse_intermediates + (size_t)head * MP + out_idx, sm->head_m[h] + mkm::log2f_exact(den));
+            if (j == 0) st_f32(a.attn_lse_intermediates + (size_t)head * MP + out_idx, m + mkm::log2f_exact(den));
         }
+        wait_stores();
+        trace_consumer(c, 28);
+        if (j == 0) signal_sharded_lane(c, layer, 2, 1);
+        trace_consumer_flush(c, 26, 28);
     }
-    wait_stores();
-    wg_barrier();
     return true;
 }
 
@@ -1428,7 +1431,7 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
         switch (opcode) {
         case 1: ok = op_qkv<KC_HID>(sm, slot, &refusal); break;
         case 2: ok = op_attention<D>(sm, slot, &refusal); break;
-        case 3: ok = op_attention_reduction(sm, slot, &refusal); break;
+        case 3: ok = op_attention_reduction<D>(sm, slot, &refusal); break;
         case 4: ok = op_matvec_add<KC_RED, false>(sm, slot, &refusal); break;
         case 5: ok = op_upgate<KC_HID>(sm, slot, &refusal); break;
         case 6: ok = op_matvec_add<KC_RED, true>(sm, slot, &refusal); break;
