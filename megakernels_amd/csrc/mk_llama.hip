@@ -60,6 +60,11 @@ constexpr int kHotRows = 4;         // barrier rows 2..5 are sharded
 constexpr int kOutRows = 2048;      // rows staged in LDS between matvec and epilogue
 constexpr int kMaxK = 4096;         // longest activation vector handed through LDS
 constexpr int kScoreCap = 4096;     // tokens per attention partition (LDS score buffer)
+#ifdef MK_NO_PAIRING
+constexpr bool kPairing = false;
+#else
+constexpr bool kPairing = true;     // run a short matvec instruction and its successor as one handler
+#endif
 constexpr int kQueueSlots = 256;    // longest instruction queue per worker (kept in LDS)
 constexpr int kMaxHeadDim = 128;
 constexpr int kGqa = 4;             // query heads per KV head handled by one attention instruction
@@ -446,14 +451,19 @@ __device__ __forceinline__ PollTicket poll_issue(const Ctx &c, const int *ptr) {
 // sum_mode: wait until the sum over lanes reaches target (sharded counter + its base value);
 // otherwise wait until every lane's counter reaches target.  Lane 63 watches the global status
 // word so that one worker's failure releases everybody.
-__device__ bool poll_wait(const Ctx &c, PollTicket t, bool sum_mode, int target) {
+// `not_yet` is called once if the first look finds the dependency unsatisfied.
+template <class NotYet>
+__device__ __forceinline__ bool poll_wait(const Ctx &c, PollTicket t, bool sum_mode, int target, NotYet not_yet) {
     const long long t0 = wall_clock64();
     const long long limit = spin_ticks(c);
     const int *status = ws_status(c);
     int v = t.value, st = t.status;
+    bool first = true;
     while (true) {
         const bool ok = sum_mode ? (lane_sum_i32(v) >= target) : (bool)__all(t.ptr == nullptr || v >= target);
         if (ok) break;
+        if (first) not_yet();
+        first = false;
         if (__any(st != 0)) return false;
         if (wall_clock64() - t0 > limit) {
             if (c.lane == 0) record_status(c, MK_STATUS_BARRIER_TIMEOUT);
@@ -466,8 +476,8 @@ __device__ bool poll_wait(const Ctx &c, PollTicket t, bool sum_mode, int target)
     compiler_fence();  // data loads stay after the successful poll
     return true;
 }
-__device__ __forceinline__ bool poll_counters(const Ctx &c, const int *ptr, bool sum_mode, int target) {
-    return poll_wait(c, poll_issue(c, ptr), sum_mode, target);
+__device__ bool poll_counters(const Ctx &c, const int *ptr, bool sum_mode, int target) {
+    return poll_wait(c, poll_issue(c, ptr), sum_mode, target, []() {});
 }
 
 __device__ __forceinline__ const int *sharded_lane_ptr(const Ctx &c, int layer, int row) {
@@ -529,10 +539,7 @@ __device__ __forceinline__ float fold8(const float (&a)[8]) {
 // Sum of squares in column order: column c = lane * 8 + e accumulates its elements j * 512 + c in
 // order of j, the 512 columns are added as a balanced pairwise tree.
 template <int KC>
-__device__ __forceinline__ void rms_norm_x(uint4 (&xq)[KC], const uint16_t *hidden, const uint4 (&wraw)[KC], float eps,
-                                           int lane) {
-    XVec<KC> x;
-    load_x<KC>(x, hidden, lane);
+__device__ __forceinline__ void rms_norm_x(uint4 (&xq)[KC], const XVec<KC> &x, const uint4 (&wraw)[KC], float eps) {
     float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
     for (int j = 0; j < KC; j++)
@@ -637,31 +644,44 @@ __device__ __forceinline__ float dot_row(const uint4 (&w)[KC], const XVec<KC> &x
 //   controller: `prepare` (wait for the dependency, build the activation vector in LDS; returns
 //               false to abandon), barrier, `overlap`, barrier, `finish` (epilogue + signal)
 // Both barriers are reached by all nine waves whatever the outcome of `prepare`.
+// The controller's side of one matvec instruction (or one batch of the LM head).
+template <class Ahead, class Prepare, class Overlap, class Finish>
+__device__ __forceinline__ bool controller_sequence(const Ctx &c, Ahead ahead, Prepare prepare, Overlap overlap,
+                                                    Finish finish) {
+    // A CU serves its memory requests in order, and the consumers' first requests are bulky.  So
+    // the controller's first requests (first look at the dependency, norm weights) go out before
+    // them, and the consumers are released (entry barrier) either when that first look says "not
+    // yet" - there is time, prefetch away - or, when the dependency is already satisfied, right
+    // after the controller has requested the activation vector.  A worker that arrives late then
+    // has its short critical requests ahead of its own prefetch instead of behind it.
+    ahead();
+    bool released = false;
+    auto release = [&]() {
+        if (!released) wg_barrier();
+        released = true;
+    };
+    const bool ok = prepare(release);
+    release();
+    trace_event(c, kEvInputReady);
+    if (!barrier_inputs_ready(c, ok)) return false;
+    overlap();  // runs while the consumers stream rows: fetch what the epilogue will need
+    wg_barrier();
+    trace_event(c, kEvComputeDone);
+    finish();
+    // the consumers hold their next requests back until the results and the signal are on their way
+    wg_barrier();
+    return true;
+}
+
+__device__ __forceinline__ int rows_of_wave(int ntasks, int wave) {
+    return ntasks > wave ? (ntasks - wave + kConsumerWaves - 1) / kConsumerWaves : 0;
+}
+
 template <int KC, int PF, class RowOf, class Ahead, class Prepare, class Overlap, class Finish>
 __device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need_x, RowOf row_ref, Ahead ahead,
                                              Prepare prepare, Overlap overlap, Finish finish) {
-    if (c.controller) {
-        // The controller's first requests: first look at the dependency, norm weights.  With
-        // MK_ENTRY_BARRIER they go out before the consumers' bulk requests (a CU serves its requests
-        // in order); measured, the activation load then queues behind the bulk instead and nothing
-        // is gained, so the barrier is off.
-        ahead();
-#ifdef MK_ENTRY_BARRIER
-        wg_barrier();
-#endif
-        const bool ok = prepare();
-        trace_event(c, kEvInputReady);
-        if (!barrier_inputs_ready(c, ok)) return false;
-        overlap();  // runs while the consumers stream rows: fetch what the epilogue will need
-        wg_barrier();
-        trace_event(c, kEvComputeDone);
-        finish();
-#ifndef MK_NO_EPILOGUE_FIRST
-        wg_barrier();
-#endif
-        return true;
-    }
-    const int mine = ntasks > c.wave ? (ntasks - c.wave + kConsumerWaves - 1) / kConsumerWaves : 0;
+    if (c.controller) return controller_sequence(c, ahead, prepare, overlap, finish);
+    const int mine = rows_of_wave(ntasks, c.wave);
     uint4 buf[PF][KC];
     // Requests are issued unconditionally wherever rows stream (rows past the end become no-op
     // requests), so the count of outstanding loads at each wait is a compile-time constant: the
@@ -674,9 +694,7 @@ __device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need
         const float y = mkm::round_bf16(dot_row<KC>(src, x));
         if (c.lane == 0) c.sm->out[c.wave + i * kConsumerWaves] = y;
     };
-#ifdef MK_ENTRY_BARRIER
-    wg_barrier();
-#endif
+    wg_barrier();  // entry: the controller's first requests are out
     trace_consumer(c, 20);
 #pragma unroll
     for (int s = 0; s < PF; s++) request(buf[s], s);
@@ -705,11 +723,9 @@ __device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need
     trace_consumer(c, 23);
     wg_barrier();
     trace_consumer_flush(c, 20, 25);
-#ifndef MK_NO_EPILOGUE_FIRST
     // hold the next instruction's weight requests back until the controller has sent this
     // instruction's results and signal: they would otherwise queue behind the bulk loads
     wg_barrier();
-#endif
     return true;
 }
 
@@ -721,38 +737,116 @@ __device__ __forceinline__ bool bail(const Ctx &c, int code, int *refusal) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// The four matvec instructions (opcodes 1, 4, 5, 6).
+//
+// describe_matvec() turns an instruction into what the consumer waves need: how many rows, and
+// where each row lives.  control_*() is the controller's side of one instruction: dependency
+// wait, activation vector into LDS, epilogue, signal.  op_matvec_chain() runs a whole run of
+// consecutive matvec instructions: the controller goes through them one by one, while each consumer
+// wave treats its rows of all of them as one stream and keeps NB row requests in flight across
+// instruction boundaries, so the next instruction's weights arrive while this one still waits for
+// its dependency or writes its results.
+// ---------------------------------------------------------------------------------------------
+struct MatvecDesc {
+    int opcode, layer, ntasks, first_row;
+    WeightBuffer w0;
+    long long gate_delta;  // opcode 5: byte distance from the up matrix (w0) to the gate matrix
+    uint32_t row_bytes;
+    InsPtr ins;
+};
+
+// false: malformed instruction (nothing has been touched)
+__device__ __forceinline__ bool describe_matvec(SmemPtr sm, int slot, MatvecDesc &d) {
+    ArgsRef a = sm->args;
+    const InsPtr ins = sm->queue[slot];
+    const int hid = uni(a.hidden_size), inter = uni(a.intermediate_size);
+    d.ins = ins;
+    d.opcode = uni(ins[0]);
+    d.layer = uni(ins[1]);
+    d.gate_delta = 0;
+    if (d.layer < 0 || d.layer >= uni(a.num_layers)) return false;
+    if (d.opcode == 1) {
+        const int start = uni(ins[2]), end = uni(ins[3]);
+        const int total_blocks = (uni(a.num_attention_heads) + 2 * uni(a.num_kv_heads)) * uni(a.head_dim) / 16;
+        if (start < 0 || end > total_blocks || end - start > kOutRows / 16) return false;
+        d.ntasks = (end > start ? end - start : 0) * 16;
+        d.first_row = start * 16;
+        d.row_bytes = (uint32_t)hid * 2u;
+        d.w0 = weight_buffer(a.qkv_weights + (size_t)d.layer * total_blocks * 16 * hid, (size_t)total_blocks * 16 * hid * 2);
+        return true;
+    }
+    if (d.opcode == 4 || d.opcode == 6) {
+        const bool is_down = d.opcode == 6;
+        const int start = uni(ins[2]), end = uni(ins[3]), group = uni(ins[4]);
+        const int R = uni(a.matvec_reduction_size), in_dim = is_down ? inter : hid;
+        if (start < 0 || end > hid / 16 || group < 0 || group >= in_dim / R || end - start > kOutRows / 16) return false;
+        d.ntasks = (end > start ? end - start : 0) * 16;
+        d.first_row = start * 16;
+        d.row_bytes = (uint32_t)in_dim * 2u;
+        // the buffer starts at this column group's first element of the layer's matrix
+        d.w0 = weight_buffer((is_down ? a.down_weights : a.o_weights) + (size_t)d.layer * hid * in_dim + (size_t)group * R,
+                             ((size_t)(hid - 1) * in_dim + R) * 2);
+        return true;
+    }
+    if (d.opcode == 5) {
+        const int n = uni(ins[2]);
+        if (n < 0 || n > MK_INSTRUCTION_WORDS - 3 || n * 32 > kOutRows) return false;
+        bool bad = false;
+        for (int i = 0; i < n; i++) bad |= ins[3 + i] < 0 || ins[3 + i] >= inter / 16;
+        if (bad) return false;
+        d.ntasks = n * 32;
+        d.first_row = 0;
+        d.row_bytes = (uint32_t)hid * 2u;
+        d.w0 = weight_buffer(a.up_weights + (size_t)d.layer * inter * hid, (size_t)inter * hid * 2);
+        const uint16_t *gate = uni(a.gate_weights + (size_t)d.layer * inter * hid);
+        d.gate_delta = (long long)((uintptr_t)gate - (uintptr_t)d.w0.base);
+        return true;
+    }
+    return false;
+}
+
+// row computed by task t of the instruction.  Opcode 5: task t is list entry t / 32, matrix
+// (t / 16) & 1 (0 up, 1 gate), row t % 16 of that block.
+__device__ __forceinline__ RowRef matvec_row(const MatvecDesc &d, int t) {
+    if (d.opcode == 5) {
+        const int blk = uni(d.ins[3 + (t >> 5)]);
+        // the gate matrix has the up matrix's size; its buffer is the up buffer moved by a distance
+        const long long shift = (t >> 4) & 1 ? d.gate_delta : 0;
+        const WeightBuffer w = {(const uint16_t *)((uintptr_t)d.w0.base + (uintptr_t)shift), d.w0.bytes};
+        return RowRef{w, (uint32_t)(blk * 16 + (t & 15)) * d.row_bytes};
+    }
+    return RowRef{d.w0, (uint32_t)(d.first_row + t) * d.row_bytes};
+}
+
+// ---------------------------------------------------------------------------------------------
 // opcode 1: RMSNorm + QKV matvec + RoPE + KV append  (python_vm.py:168-248;
 // reference device op: demos/low-latency-llama/rms_matvec_rope_append.cu:10-231)
 // ---------------------------------------------------------------------------------------------
 template <int KC>
-static __device__ __noinline__ bool op_qkv(SmemPtr lds, int slot, int *refusal) {
-    const InsPtr ins = lds->queue[slot];
-    const Ctx c = make_ctx(lds, slot, ins[0]);
+__device__ __forceinline__ bool control_qkv(const Ctx &c) {
+    const InsPtr ins = c.sm->queue[c.slot];
     ArgsRef a = c.sm->args;
     const int layer = ins[1], start = ins[2], end = ins[3];
     const int hid = a.hidden_size, D = a.head_dim, H = a.num_attention_heads, KVH = a.num_kv_heads;
-    const int total_blocks = (H + 2 * KVH) * D / 16;
-    if (layer < 0 || layer >= a.num_layers || start < 0 || end > total_blocks || end - start > kOutRows / 16)
-        return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
     const int nblk = end > start ? end - start : 0;
-    const size_t matrix_bytes = (size_t)total_blocks * 16 * hid * 2;
-    const WeightBuffer W = weight_buffer(a.qkv_weights + (size_t)layer * total_blocks * 16 * hid, matrix_bytes);
     const int down_jobs = (a.intermediate_size / a.matvec_reduction_size) * (hid / 16);
     PollTicket ticket = {nullptr, 0, 0};
     uint4 wraw[KC];
-
-    return matvec_batch<KC, rows_in_flight<KC>(MK_PF_QKV)>(
-        c, nblk * 16, nblk > 0, [&](int t) { return RowRef{W, (uint32_t)(start * 16 + t) * (uint32_t)hid * 2u}; },
+    return controller_sequence(
+        c,
         [&]() {
             if (layer > 0) ticket = poll_issue(c, sharded_lane_ptr(c, layer - 1, 5));
             if (nblk > 0) load_row<KC>(wraw, a.attn_norm_weights + (size_t)layer * hid, c.lane);
         },
-        [&]() {
-            if (layer > 0 && !poll_wait(c, ticket, true, down_jobs)) return false;
+        [&](auto release) {
+            if (layer > 0 && !poll_wait(c, ticket, true, down_jobs, release)) return false;
             trace_event(c, kEvDepReady);
             if (nblk > 0) {
+                XVec<KC> x;
+                load_x<KC>(x, a.hidden_states, c.lane);
+                release();
                 uint4 xq[KC];
-                rms_norm_x<KC>(xq, a.hidden_states, wraw, a.rms_norm_eps, c.lane);
+                rms_norm_x<KC>(xq, x, wraw, a.rms_norm_eps);
                 x_to_lds<KC>(xq, c.sm, c.lane);
             }
             return true;
@@ -798,22 +892,14 @@ static __device__ __noinline__ bool op_qkv(SmemPtr lds, int slot, int *refusal) 
 // rounding chain is reproduced without serialising the workers.
 // ---------------------------------------------------------------------------------------------
 template <int KC, bool is_down>
-static __device__ __noinline__ bool op_matvec_add(SmemPtr lds, int slot, int *refusal) {
-    const InsPtr ins = lds->queue[slot];
-    const Ctx c = make_ctx(lds, slot, ins[0]);
+__device__ __forceinline__ bool control_matvec_add(const Ctx &c) {
+    const InsPtr ins = c.sm->queue[c.slot];
     ArgsRef a = c.sm->args;
     const int layer = ins[1], start = ins[2], end = ins[3], group = ins[4];
     const int hid = a.hidden_size, R = a.matvec_reduction_size;
     const int in_dim = is_down ? a.intermediate_size : hid;
     const int ngroups = in_dim / R;
-    if (layer < 0 || layer >= a.num_layers || start < 0 || end > hid / 16 || group < 0 || group >= ngroups ||
-        end - start > kOutRows / 16)
-        return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
     const int nblk = end > start ? end - start : 0;
-    // the buffer starts at this column group's first element of the layer's matrix
-    const WeightBuffer W =
-        weight_buffer((is_down ? a.down_weights : a.o_weights) + (size_t)layer * hid * in_dim + (size_t)group * R,
-                      ((size_t)(hid - 1) * in_dim + R) * 2);
     const uint16_t *vec = (is_down ? a.silu_out : a.attn_out) + (size_t)group * R;
     const int wait_row = is_down ? 4 : 2;
     const int wait_target = is_down ? a.intermediate_size / 16 : a.num_attention_heads;
@@ -824,16 +910,16 @@ static __device__ __noinline__ bool op_matvec_add(SmemPtr lds, int slot, int *re
     uint32_t pre[kPre] = {0, 0};
     const bool prefetched = nblk * 8 <= kPre * 64;
     PollTicket ticket = {nullptr, 0, 0};
-
-    return matvec_batch<KC, rows_in_flight<KC>(is_down ? MK_PF_DOWN : MK_PF_OPROJ)>(
-        c, nblk * 16, nblk > 0, [&](int t) { return RowRef{W, (uint32_t)(start * 16 + t) * (uint32_t)in_dim * 2u}; },
+    return controller_sequence(
+        c,
         [&]() { ticket = poll_issue(c, sharded_lane_ptr(c, layer, wait_row)); },
-        [&]() {
-            if (!poll_wait(c, ticket, true, wait_target)) return false;
+        [&](auto release) {
+            if (!poll_wait(c, ticket, true, wait_target, release)) return false;
             trace_event(c, kEvDepReady);
             if (nblk > 0) {
                 uint4 xq[KC];
                 load_xq<KC>(xq, vec, c.lane);
+                release();
                 x_to_lds<KC>(xq, c.sm, c.lane);
             }
             return true;
@@ -892,40 +978,29 @@ static __device__ __noinline__ bool op_matvec_add(SmemPtr lds, int slot, int *re
 // reference device op: demos/low-latency-llama/upgate.cu:10-172)
 // ---------------------------------------------------------------------------------------------
 template <int KC>
-static __device__ __noinline__ bool op_upgate(SmemPtr lds, int slot, int *refusal) {
-    const InsPtr ins = lds->queue[slot];
-    const Ctx c = make_ctx(lds, slot, ins[0]);
+__device__ __forceinline__ bool control_upgate(const Ctx &c) {
+    const InsPtr ins = c.sm->queue[c.slot];
     ArgsRef a = c.sm->args;
     const int layer = ins[1], n = ins[2];
-    const int hid = a.hidden_size, inter = a.intermediate_size;
-    bool bad = layer < 0 || layer >= a.num_layers || n < 0 || n > MK_INSTRUCTION_WORDS - 3 || n * 32 > kOutRows;
-    if (!bad)
-        for (int i = 0; i < n; i++) bad |= ins[3 + i] < 0 || ins[3 + i] >= inter / 16;
-    if (bad) return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
-    const size_t matrix_bytes = (size_t)inter * hid * 2;
-    const WeightBuffer Wu = weight_buffer(a.up_weights + (size_t)layer * inter * hid, matrix_bytes);
-    const WeightBuffer Wg = weight_buffer(a.gate_weights + (size_t)layer * inter * hid, matrix_bytes);
+    const int hid = a.hidden_size;
     const int o_jobs = (hid / a.matvec_reduction_size) * (hid / 16);
     PollTicket ticket = {nullptr, 0, 0};
     uint4 wraw[KC];
-
-    // task t: list entry t / 32, matrix (t / 16) & 1 (0 up, 1 gate), row t % 16
-    return matvec_batch<KC, rows_in_flight<KC>(MK_PF_UPGATE)>(
-        c, n * 32, n > 0,
-        [&](int t) {
-            const int blk = ins[3 + (t >> 5)];
-            return RowRef{(t >> 4) & 1 ? Wg : Wu, (uint32_t)(blk * 16 + (t & 15)) * (uint32_t)hid * 2u};
-        },
+    return controller_sequence(
+        c,
         [&]() {
             ticket = poll_issue(c, sharded_lane_ptr(c, layer, 3));
             if (n > 0) load_row<KC>(wraw, a.mlp_norm_weights + (size_t)layer * hid, c.lane);
         },
-        [&]() {
-            if (!poll_wait(c, ticket, true, o_jobs)) return false;
+        [&](auto release) {
+            if (!poll_wait(c, ticket, true, o_jobs, release)) return false;
             trace_event(c, kEvDepReady);
             if (n > 0) {
+                XVec<KC> x;
+                load_x<KC>(x, a.hidden_states, c.lane);
+                release();
                 uint4 xq[KC];
-                rms_norm_x<KC>(xq, a.hidden_states, wraw, a.rms_norm_eps, c.lane);
+                rms_norm_x<KC>(xq, x, wraw, a.rms_norm_eps);
                 x_to_lds<KC>(xq, c.sm, c.lane);
             }
             return true;
@@ -943,6 +1018,123 @@ static __device__ __noinline__ bool op_upgate(SmemPtr lds, int slot, int *refusa
             wait_stores();
             signal_sharded(c, layer, 4, n);
         });
+}
+
+// ---------------------------------------------------------------------------------------------
+// Consumer side of one matvec instruction, in two parts, so that the first rows of the instruction
+// that follows can be requested in between.  Wave w computes tasks w, w + 8, ...; PF rows are in
+// flight.  Requests are issued unconditionally wherever rows stream (rows past the end become no-op
+// requests), so the count of outstanding loads at each wait is a compile-time constant.
+// ---------------------------------------------------------------------------------------------
+template <int KC, int PF>
+__device__ __forceinline__ void consumer_request_first(const Ctx &c, uint4 (&buf)[PF][KC], const MatvecDesc &d, int mine) {
+#pragma unroll
+    for (int s = 0; s < PF; s++) load_row<KC>(buf[s], matvec_row(d, c.wave + s * kConsumerWaves), s < mine, c.lane);
+}
+
+template <int KC, int PF>
+__device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&buf)[PF][KC], const MatvecDesc &d, int mine) {
+    if (!barrier_inputs_ready(c, true)) return false;
+    trace_consumer(c, 22);
+    XVec<KC> x;
+    if (d.ntasks > 0) x_from_lds<KC>(x, c.sm, c.lane);
+    trace_consumer(c, 24);
+    auto consume = [&](const uint4 (&src)[KC], int i) {
+        const float y = mkm::round_bf16(dot_row<KC>(src, x));
+        if (c.lane == 0) c.sm->out[c.wave + i * kConsumerWaves] = y;
+    };
+    int base = 0;
+    // rounds that are followed by more rows: every row of the round exists, every buffer is refilled
+    for (; base + PF < mine; base += PF) {
+#pragma unroll
+        for (int s = 0; s < PF; s++) {
+            consume(buf[s], base + s);
+            compiler_fence();
+            const int i = base + s + PF;
+            load_row<KC>(buf[s], matvec_row(d, c.wave + i * kConsumerWaves), i < mine, c.lane);
+            compiler_fence();
+        }
+    }
+    trace_consumer(c, 25);
+    // last round: nothing left to request
+#pragma unroll
+    for (int s = 0; s < PF; s++)
+        if (base + s < mine) consume(buf[s], base + s);
+    trace_consumer(c, 23);
+    wg_barrier();  // results are in LDS
+    // hold further weight requests back until the controller has sent this instruction's results and
+    // signal: they would otherwise queue behind the bulk loads
+    wg_barrier();
+    return true;
+}
+
+template <int KC>
+__device__ __forceinline__ bool control_matvec(const Ctx &c) {
+    switch (c.opcode) {
+    case 1: return control_qkv<KC>(c);
+    case 4: return control_matvec_add<KC, false>(c);
+    case 5: return control_upgate<KC>(c);
+    default: return control_matvec_add<KC, true>(c);
+    }
+}
+
+__device__ __forceinline__ constexpr int pf_of(int opcode) {
+    return opcode == 1 ? MK_PF_QKV : opcode == 4 ? MK_PF_OPROJ : opcode == 5 ? MK_PF_UPGATE : MK_PF_DOWN;
+}
+
+// One matvec instruction (opcode OP, row width KC chunks).
+template <int OP, int KC>
+static __device__ __noinline__ bool op_matvec(SmemPtr lds, int slot, int *refusal) {
+    constexpr int PF = rows_in_flight<KC>(pf_of(OP));
+    const Ctx c = make_ctx(lds, slot, OP);
+    MatvecDesc d;
+    if (!describe_matvec(lds, slot, d)) return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
+    if (c.controller) return control_matvec<KC>(c);
+    const int mine = rows_of_wave(d.ntasks, c.wave);
+    uint4 buf[PF][KC];
+    wg_barrier();  // entry: the controller's first requests are out
+    trace_consumer(c, 20);
+    consumer_request_first<KC, PF>(c, buf, d, mine);
+    trace_consumer(c, 21);
+    const bool ok = consumer_run<KC, PF>(c, buf, d, mine);
+    trace_consumer_flush(c, 20, 25);
+    return ok;
+}
+
+// Two matvec instructions in a row (opcodes OP_A, OP_B) whose first is short: the second one's first
+// rows are requested together with the first one's, so they arrive while the first instruction
+// waits for its dependency instead of after it.  The caller has checked the second opcode.
+// Returns the number of instructions executed (2, or 1 when the second one is malformed and left
+// to report itself), 0 on failure.
+template <int OP_A, int KC_A, int OP_B, int KC_B>
+static __device__ __noinline__ int op_matvec_pair(SmemPtr lds, int slot, int *refusal) {
+    constexpr int PF_A = rows_in_flight<KC_A>(pf_of(OP_A)), PF_B = rows_in_flight<KC_B>(pf_of(OP_B));
+    const Ctx ca = make_ctx(lds, slot, OP_A);
+    const Ctx cb = make_ctx(lds, slot + 1, OP_B);
+    MatvecDesc da, db;
+    if (!describe_matvec(lds, slot, da)) {
+        bail(ca, MK_STATUS_BAD_INSTRUCTION, refusal);
+        return 0;
+    }
+    const bool pair = describe_matvec(lds, slot + 1, db);
+    if (ca.controller) {
+        if (!control_matvec<KC_A>(ca)) return 0;
+        if (!pair) return 1;
+        trace_event(ca, kEvEnd);
+        trace_event(cb, kEvStart);
+        if (cb.trace && cb.lane == 0) st_plain_i32(cb.trace + kEvOpcode, OP_B);
+        return control_matvec<KC_B>(cb) ? 2 : 0;
+    }
+    const int mine_a = rows_of_wave(da.ntasks, ca.wave);
+    const int mine_b = pair ? rows_of_wave(db.ntasks, ca.wave) : 0;
+    uint4 buf_a[PF_A][KC_A], buf_b[PF_B][KC_B];
+    wg_barrier();  // entry of the first instruction
+    consumer_request_first<KC_A, PF_A>(ca, buf_a, da, mine_a);
+    if (pair) consumer_request_first<KC_B, PF_B>(cb, buf_b, db, mine_b);
+    if (!consumer_run<KC_A, PF_A>(ca, buf_a, da, mine_a)) return 0;
+    if (!pair) return 1;
+    wg_barrier();  // entry of the second instruction: its requests went out long ago
+    return consumer_run<KC_B, PF_B>(cb, buf_b, db, mine_b) ? 2 : 0;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -974,12 +1166,15 @@ static __device__ __noinline__ bool op_lm_head(SmemPtr lds, int slot, int *refus
                 ticket = poll_issue(c, sharded_lane_ptr(c, a.num_layers - 1, 5));
                 load_row<KC>(wraw, a.lm_head_norm_weights, c.lane);
             },
-            [&]() {
+            [&](auto release) {
                 if (!first) return true;  // the activation vector stays in LDS between batches
-                if (!poll_wait(c, ticket, true, down_jobs)) return false;
+                if (!poll_wait(c, ticket, true, down_jobs, release)) return false;
                 trace_event(c, kEvDepReady);
+                XVec<KC> x;
+                load_x<KC>(x, a.hidden_states, c.lane);
+                release();
                 uint4 xq[KC];
-                rms_norm_x<KC>(xq, a.hidden_states, wraw, a.rms_norm_eps, c.lane);
+                rms_norm_x<KC>(xq, x, wraw, a.rms_norm_eps);
                 x_to_lds<KC>(xq, c.sm, c.lane);
                 return true;
             },
@@ -1428,18 +1623,36 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
             if (c.trace && c.controller && c.lane == 0) st_plain_i32(c.trace + kEvOpcode, opcode);
         }
         bool ok = true;
+        int executed = 1;  // queue slots the handler went through
+        const int next_opcode = slot + 1 < a.num_slots ? sm->queue[slot + 1][0] : 0;
         switch (opcode) {
-        case 1: ok = op_qkv<KC_HID>(sm, slot, &refusal); break;
+        case 1: ok = op_matvec<1, KC_HID>(sm, slot, &refusal); break;
         case 2: ok = op_attention<D>(sm, slot, &refusal); break;
         case 3: ok = op_attention_reduction<D>(sm, slot, &refusal); break;
-        case 4: ok = op_matvec_add<KC_RED, false>(sm, slot, &refusal); break;
-        case 5: ok = op_upgate<KC_HID>(sm, slot, &refusal); break;
-        case 6: ok = op_matvec_add<KC_RED, true>(sm, slot, &refusal); break;
+        case 4:
+            // a short instruction with a long wait: fetch the next one's first rows meanwhile
+            if (kPairing && next_opcode == 5) {
+                executed = op_matvec_pair<4, KC_RED, 5, KC_HID>(sm, slot, &refusal);
+                ok = executed > 0;
+            } else {
+                ok = op_matvec<4, KC_RED>(sm, slot, &refusal);
+            }
+            break;
+        case 5: ok = op_matvec<5, KC_HID>(sm, slot, &refusal); break;
+        case 6:
+            if (kPairing && next_opcode == 1) {
+                executed = op_matvec_pair<6, KC_RED, 1, KC_HID>(sm, slot, &refusal);
+                ok = executed > 0;
+            } else {
+                ok = op_matvec<6, KC_RED>(sm, slot, &refusal);
+            }
+            break;
         case 7: ok = op_lm_head<KC_HID>(sm, slot, &refusal); break;
         default: ok = bail(make_ctx(sm, slot, opcode), MK_STATUS_BAD_OPCODE, &refusal);  // reference: trap, include/util.cuh:38
         }
-        trace_event(make_ctx(sm, slot, opcode), kEvEnd);
         if (!ok) break;
+        slot += executed - 1;
+        trace_event(make_ctx(sm, slot, sm->queue[slot][0]), kEvEnd);
     }
     if (refusal && tid == 0) sm->abort = refusal;
 
