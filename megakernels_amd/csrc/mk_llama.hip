@@ -39,6 +39,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <type_traits>
 
 #include "../../include/mk_llama.h"
 #include "mk_math.h"
@@ -60,11 +61,6 @@ constexpr int kHotRows = 4;         // barrier rows 2..5 are sharded
 constexpr int kOutRows = 2048;      // rows staged in LDS between matvec and epilogue
 constexpr int kMaxK = 4096;         // longest activation vector handed through LDS
 constexpr int kScoreCap = 4096;     // tokens per attention partition (LDS score buffer)
-#ifdef MK_NO_PAIRING
-constexpr bool kPairing = false;
-#else
-constexpr bool kPairing = true;     // run a short matvec instruction and its successor as one handler
-#endif
 constexpr int kQueueSlots = 256;    // longest instruction queue per worker (kept in LDS)
 constexpr int kMaxHeadDim = 128;
 constexpr int kGqa = 4;             // query heads per KV head handled by one attention instruction
@@ -82,10 +78,10 @@ constexpr int kDoneSlot = 8;        // workspace int: workgroups finished
 #define MK_PF_OPROJ 2
 #endif
 #ifndef MK_PF_UPGATE
-#define MK_PF_UPGATE 4
+#define MK_PF_UPGATE 5
 #endif
 #ifndef MK_PF_DOWN
-#define MK_PF_DOWN 4
+#define MK_PF_DOWN 3
 #endif
 #ifndef MK_PF_LMHEAD
 #define MK_PF_LMHEAD 4
@@ -655,7 +651,12 @@ __device__ __forceinline__ bool controller_sequence(const Ctx &c, Ahead ahead, P
     // after the controller has requested the activation vector.  A worker that arrives late then
     // has its short critical requests ahead of its own prefetch instead of behind it.
     ahead();
+#ifdef MK_NO_GATE
+    bool released = true;
+    wg_barrier();
+#else
     bool released = false;
+#endif
     auto release = [&]() {
         if (!released) wg_barrier();
         released = true;
@@ -741,11 +742,12 @@ __device__ __forceinline__ bool bail(const Ctx &c, int code, int *refusal) {
 //
 // describe_matvec() turns an instruction into what the consumer waves need: how many rows, and
 // where each row lives.  control_*() is the controller's side of one instruction: dependency
-// wait, activation vector into LDS, epilogue, signal.  op_matvec_chain() runs a whole run of
-// consecutive matvec instructions: the controller goes through them one by one, while each consumer
-// wave treats its rows of all of them as one stream and keeps NB row requests in flight across
-// instruction boundaries, so the next instruction's weights arrive while this one still waits for
-// its dependency or writes its results.
+// wait, activation vector into LDS, epilogue, signal.  op_matvec() is the handler: the consumer
+// waves request their first rows on entry (the prefetch that overlaps the dependency wait), then
+// stream the rest.  (Requesting rows of the *following* instructions as well - a row stream across
+// instruction boundaries, or up/gate, down and QKV rows fetched while attention runs - was built
+// and measured: the bulk requests delay the short latency-critical ones of the instructions in
+// between, and a decode step got 5 % slower.)
 // ---------------------------------------------------------------------------------------------
 struct MatvecDesc {
     int opcode, layer, ntasks, first_row;
@@ -1021,19 +1023,38 @@ __device__ __forceinline__ bool control_upgate(const Ctx &c) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Consumer side of one matvec instruction, in two parts, so that the first rows of the instruction
-// that follows can be requested in between.  Wave w computes tasks w, w + 8, ...; PF rows are in
-// flight.  Requests are issued unconditionally wherever rows stream (rows past the end become no-op
-// requests), so the count of outstanding loads at each wait is a compile-time constant.
+// Consumer side of the matvec instructions.  Wave w computes tasks w, w + 8, ... of an instruction.
+// Weight rows travel through a pool of row buffers (registers); which buffers an instruction uses,
+// in which order, is a compile-time list (BufMap), so all register indexing is static.  Requests are
+// issued unconditionally (rows past the end become no-op requests): the count of outstanding loads
+// at each wait is then a compile-time constant, also across the instructions that one handler
+// executes in a row.
 // ---------------------------------------------------------------------------------------------
-template <int KC, int PF>
-__device__ __forceinline__ void consumer_request_first(const Ctx &c, uint4 (&buf)[PF][KC], const MatvecDesc &d, int mine) {
+template <int... IDX>
+struct BufMap {
+    static constexpr int size = sizeof...(IDX);
+    static constexpr int at(int s) {
+        constexpr int idx[] = {IDX...};
+        return idx[s];
+    }
+};
+
+// request rows first, first + 1, ... of this wave into the buffers of the list (`present` false:
+// the instruction is not there, all requests are no-ops)
+template <int KC, class Map, int NBUF>
+__device__ __forceinline__ void request_rows(const Ctx &c, uint4 (&pool)[NBUF][KC], const MatvecDesc &d, int first, int mine,
+                                             bool present = true) {
 #pragma unroll
-    for (int s = 0; s < PF; s++) load_row<KC>(buf[s], matvec_row(d, c.wave + s * kConsumerWaves), s < mine, c.lane);
+    for (int s = 0; s < Map::size; s++)
+        load_row<KC>(pool[Map::at(s)], matvec_row(d, c.wave + (first + s) * kConsumerWaves), present && first + s < mine, c.lane);
 }
 
-template <int KC, int PF>
-__device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&buf)[PF][KC], const MatvecDesc &d, int mine) {
+// One instruction, its first Map::size rows already requested into the listed buffers: wait for the
+// activation vector, stream the rows (Map::size in flight), leave the results in LDS, and wait until
+// the controller has sent them.
+template <int KC, class Map, int NBUF>
+__device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&pool)[NBUF][KC], const MatvecDesc &d, int mine) {
+    constexpr int PF = Map::size;
     if (!barrier_inputs_ready(c, true)) return false;
     trace_consumer(c, 22);
     XVec<KC> x;
@@ -1048,10 +1069,10 @@ __device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&buf)[PF][KC],
     for (; base + PF < mine; base += PF) {
 #pragma unroll
         for (int s = 0; s < PF; s++) {
-            consume(buf[s], base + s);
+            consume(pool[Map::at(s)], base + s);
             compiler_fence();
             const int i = base + s + PF;
-            load_row<KC>(buf[s], matvec_row(d, c.wave + i * kConsumerWaves), i < mine, c.lane);
+            load_row<KC>(pool[Map::at(s)], matvec_row(d, c.wave + i * kConsumerWaves), i < mine, c.lane);
             compiler_fence();
         }
     }
@@ -1059,7 +1080,7 @@ __device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&buf)[PF][KC],
     // last round: nothing left to request
 #pragma unroll
     for (int s = 0; s < PF; s++)
-        if (base + s < mine) consume(buf[s], base + s);
+        if (base + s < mine) consume(pool[Map::at(s)], base + s);
     trace_consumer(c, 23);
     wg_barrier();  // results are in LDS
     // hold further weight requests back until the controller has sent this instruction's results and
@@ -1081,60 +1102,33 @@ __device__ __forceinline__ bool control_matvec(const Ctx &c) {
 __device__ __forceinline__ constexpr int pf_of(int opcode) {
     return opcode == 1 ? MK_PF_QKV : opcode == 4 ? MK_PF_OPROJ : opcode == 5 ? MK_PF_UPGATE : MK_PF_DOWN;
 }
+template <int N>
+struct FirstBuffers;  // BufMap<0, 1, ..., N - 1>
+template <> struct FirstBuffers<1> { typedef BufMap<0> type; };
+template <> struct FirstBuffers<2> { typedef BufMap<0, 1> type; };
+template <> struct FirstBuffers<3> { typedef BufMap<0, 1, 2> type; };
+template <> struct FirstBuffers<4> { typedef BufMap<0, 1, 2, 3> type; };
+template <> struct FirstBuffers<5> { typedef BufMap<0, 1, 2, 3, 4> type; };
+template <> struct FirstBuffers<6> { typedef BufMap<0, 1, 2, 3, 4, 5> type; };
 
 // One matvec instruction (opcode OP, row width KC chunks).
 template <int OP, int KC>
 static __device__ __noinline__ bool op_matvec(SmemPtr lds, int slot, int *refusal) {
     constexpr int PF = rows_in_flight<KC>(pf_of(OP));
+    typedef typename FirstBuffers<PF>::type Map;
     const Ctx c = make_ctx(lds, slot, OP);
     MatvecDesc d;
     if (!describe_matvec(lds, slot, d)) return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
     if (c.controller) return control_matvec<KC>(c);
     const int mine = rows_of_wave(d.ntasks, c.wave);
-    uint4 buf[PF][KC];
+    uint4 pool[PF][KC];
     wg_barrier();  // entry: the controller's first requests are out
     trace_consumer(c, 20);
-    consumer_request_first<KC, PF>(c, buf, d, mine);
+    request_rows<KC, Map>(c, pool, d, 0, mine);
     trace_consumer(c, 21);
-    const bool ok = consumer_run<KC, PF>(c, buf, d, mine);
+    const bool ok = consumer_run<KC, Map>(c, pool, d, mine);
     trace_consumer_flush(c, 20, 25);
     return ok;
-}
-
-// Two matvec instructions in a row (opcodes OP_A, OP_B) whose first is short: the second one's first
-// rows are requested together with the first one's, so they arrive while the first instruction
-// waits for its dependency instead of after it.  The caller has checked the second opcode.
-// Returns the number of instructions executed (2, or 1 when the second one is malformed and left
-// to report itself), 0 on failure.
-template <int OP_A, int KC_A, int OP_B, int KC_B>
-static __device__ __noinline__ int op_matvec_pair(SmemPtr lds, int slot, int *refusal) {
-    constexpr int PF_A = rows_in_flight<KC_A>(pf_of(OP_A)), PF_B = rows_in_flight<KC_B>(pf_of(OP_B));
-    const Ctx ca = make_ctx(lds, slot, OP_A);
-    const Ctx cb = make_ctx(lds, slot + 1, OP_B);
-    MatvecDesc da, db;
-    if (!describe_matvec(lds, slot, da)) {
-        bail(ca, MK_STATUS_BAD_INSTRUCTION, refusal);
-        return 0;
-    }
-    const bool pair = describe_matvec(lds, slot + 1, db);
-    if (ca.controller) {
-        if (!control_matvec<KC_A>(ca)) return 0;
-        if (!pair) return 1;
-        trace_event(ca, kEvEnd);
-        trace_event(cb, kEvStart);
-        if (cb.trace && cb.lane == 0) st_plain_i32(cb.trace + kEvOpcode, OP_B);
-        return control_matvec<KC_B>(cb) ? 2 : 0;
-    }
-    const int mine_a = rows_of_wave(da.ntasks, ca.wave);
-    const int mine_b = pair ? rows_of_wave(db.ntasks, ca.wave) : 0;
-    uint4 buf_a[PF_A][KC_A], buf_b[PF_B][KC_B];
-    wg_barrier();  // entry of the first instruction
-    consumer_request_first<KC_A, PF_A>(ca, buf_a, da, mine_a);
-    if (pair) consumer_request_first<KC_B, PF_B>(cb, buf_b, db, mine_b);
-    if (!consumer_run<KC_A, PF_A>(ca, buf_a, da, mine_a)) return 0;
-    if (!pair) return 1;
-    wg_barrier();  // entry of the second instruction: its requests went out long ago
-    return consumer_run<KC_B, PF_B>(cb, buf_b, db, mine_b) ? 2 : 0;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1623,36 +1617,18 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
             if (c.trace && c.controller && c.lane == 0) st_plain_i32(c.trace + kEvOpcode, opcode);
         }
         bool ok = true;
-        int executed = 1;  // queue slots the handler went through
-        const int next_opcode = slot + 1 < a.num_slots ? sm->queue[slot + 1][0] : 0;
         switch (opcode) {
         case 1: ok = op_matvec<1, KC_HID>(sm, slot, &refusal); break;
         case 2: ok = op_attention<D>(sm, slot, &refusal); break;
         case 3: ok = op_attention_reduction<D>(sm, slot, &refusal); break;
-        case 4:
-            // a short instruction with a long wait: fetch the next one's first rows meanwhile
-            if (kPairing && next_opcode == 5) {
-                executed = op_matvec_pair<4, KC_RED, 5, KC_HID>(sm, slot, &refusal);
-                ok = executed > 0;
-            } else {
-                ok = op_matvec<4, KC_RED>(sm, slot, &refusal);
-            }
-            break;
+        case 4: ok = op_matvec<4, KC_RED>(sm, slot, &refusal); break;
         case 5: ok = op_matvec<5, KC_HID>(sm, slot, &refusal); break;
-        case 6:
-            if (kPairing && next_opcode == 1) {
-                executed = op_matvec_pair<6, KC_RED, 1, KC_HID>(sm, slot, &refusal);
-                ok = executed > 0;
-            } else {
-                ok = op_matvec<6, KC_RED>(sm, slot, &refusal);
-            }
-            break;
+        case 6: ok = op_matvec<6, KC_RED>(sm, slot, &refusal); break;
         case 7: ok = op_lm_head<KC_HID>(sm, slot, &refusal); break;
         default: ok = bail(make_ctx(sm, slot, opcode), MK_STATUS_BAD_OPCODE, &refusal);  // reference: trap, include/util.cuh:38
         }
         if (!ok) break;
-        slot += executed - 1;
-        trace_event(make_ctx(sm, slot, sm->queue[slot][0]), kEvEnd);
+        trace_event(make_ctx(sm, slot, opcode), kEvEnd);
     }
     if (refusal && tid == 0) sm->abort = refusal;
 
