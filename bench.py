@@ -3,9 +3,11 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2]
 
 One "step" is one decode step (one token): embedding row -> hidden state,
-barrier reset, ONE megakernel launch, argmax over the logits, token write -
+barrier reset, the instruction stream, argmax over the logits, token write -
 the per-token loop of the reference's mk generator
-(megakernels/generators.py:121-163).  Weights, KV cache and instruction
+(megakernels/generators.py:121-163).  By default all of it is ONE megakernel
+launch (--loop fused); --loop reference runs the reference's sequence of small
+kernels around the launch instead.  Weights, KV cache and instruction
 tensor are resident in HBM before the timed region starts.
 
 Workloads (all Llama-3.2-1B architecture, random bf16 weights N(0, 0.02) from
@@ -59,6 +61,10 @@ def main():
     ap.add_argument("--cpu-steps", type=int, default=32, help="decode steps timed on the CPU checker (0 = skip)")
     ap.add_argument("--sched", default="rr")
     ap.add_argument("--partitions", type=int, default=0, help="attention partitions (0 = one per 256 positions, max 24)")
+    ap.add_argument("--loop", default="fused", choices=["fused", "reference"],
+                    help="fused: one launch per token (embedding row, barrier reset and argmax inside the "
+                         "megakernel); reference: the reference generator's sequence of small kernels around "
+                         "the launch")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="after the timed region also run a plain 1 GiB device copy three times, so that a "
                          "rocprofv3 --pmc run of this command holds a kernel of known traffic to scale "
@@ -117,7 +123,7 @@ def main():
     schedule = LatencyScheduleBuilder.build(model, num_attention_partitions=partitions)
     tensorize_instructions(schedule.globs, assign_to_sms(args.sched, schedule=schedule))
     interpreter = make_mk_interpreter("latency")
-    gen = MK_Generator(model, interpreter, schedule)
+    gen = MK_Generator(model, interpreter, schedule, fused_step=args.loop == "fused")
     mk_mod = sys.modules["mk_llama"]
 
     ntok = total_steps + 1
@@ -137,22 +143,24 @@ def main():
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
     counter = {"i": 0}
-    plain_interpret = interpreter.interpret
+    plain_interpret, plain_step = interpreter.interpret, interpreter.interpret_step
 
-    def timed_interpret(globs):
-        i = counter["i"]
-        starts[i].record()
-        plain_interpret(globs)
-        ends[i].record()
-        counter["i"] = i + 1
+    def timed(launch):
+        def wrapper(*a, **kw):
+            i = counter["i"]
+            starts[i].record()
+            launch(*a, **kw)
+            ends[i].record()
+            counter["i"] = i + 1
+        return wrapper
 
-    interpreter.interpret = timed_interpret
+    interpreter.interpret, interpreter.interpret_step = timed(plain_interpret), timed(plain_step)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     gen.generate(output_tokens, prompt_len=prefill, ntok=args.steps, ntok_already_generated=1 + args.warmup)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    interpreter.interpret = plain_interpret
+    interpreter.interpret, interpreter.interpret_step = plain_interpret, plain_step
     mk_mod.check_status(device)
 
     kernel_ms = [s.elapsed_time(e) for s, e in zip(starts, ends)]
@@ -227,6 +235,7 @@ def main():
             "workers": workers,
             "attention_partitions": partitions,
             "assignment": args.sched,
+            "loop": args.loop,
             "instructions_per_step": len(schedule.dag_nodes),
         },
         "roofline": {

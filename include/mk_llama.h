@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define MK_LLAMA_ABI_VERSION 1
+#define MK_LLAMA_ABI_VERSION 2
 #define MK_INSTRUCTION_WORDS 32   /* megakernels/scheduler.py:13, include/config.cuh:14 */
 #define MK_TIMING_SLOTS 128       /* megakernels/scheduler.py:14, include/config.cuh:18 */
 #define MK_BARRIER_ROWS 10        /* megakernels/demos/latency/scheduler.py:53-61 */
@@ -31,6 +31,10 @@ extern "C" {
  * 2 matvec done, 3 end - ticks of the 100 MHz wall clock since the workgroup started; slot 4 opcode).
  * Counterpart of the reference's compile-time TIMING_RECORD_ENABLED (include/config.cuh:46). */
 #define MK_FLAG_TIMINGS 1u
+/* args.flags: leave `barriers` all zero after the launch instead of holding the VM's counts, so that
+ * the next launch needs no reset (the reference's loop refills the tensor before every launch,
+ * megakernels/generators.py:127-128). */
+#define MK_FLAG_RESET_BARRIERS 2u
 
 /* Status codes written by the kernel into the workspace and returned by
  * mk_llama_read_status(). */
@@ -39,7 +43,8 @@ enum {
     MK_STATUS_BARRIER_TIMEOUT = 1,   /* a barrier wait exceeded spin_limit_us */
     MK_STATUS_BAD_OPCODE = 2,        /* reference: asm trap, include/util.cuh:38 */
     MK_STATUS_ATTN_TOO_LONG = 3,     /* one attention partition exceeds the on-chip score buffer */
-    MK_STATUS_BAD_INSTRUCTION = 4    /* field out of range for the given shapes */
+    MK_STATUS_BAD_INSTRUCTION = 4,   /* field out of range for the given shapes */
+    MK_STATUS_BAD_TOKEN = 5          /* *token_in outside the vocabulary */
 };
 
 /* Arguments of one launch, in the positional order of the reference binding
@@ -89,6 +94,12 @@ typedef struct mk_llama_args {
     uint64_t workspace_bytes;
     uint32_t spin_limit_us;               /* give up a barrier wait after this long; 0 = default (2 s) */
     uint32_t flags;                       /* MK_FLAG_* */
+    /* Optional: the per-token glue of the reference's decode loop folded into the launch
+     * (megakernels/generators.py:121-143: embedding row -> hidden_states before the launch,
+     * argmax(logits) after it).  All NULL gives exactly the reference call. */
+    const uint16_t *embed_table;          /* [vocab, hidden]; needed with token_in */
+    const int64_t *token_in;              /* device; hidden_states starts as embed_table[*token_in] */
+    int64_t *token_out;                   /* device; receives argmax(logits), first index on ties */
 } mk_llama_args;
 
 /* Bytes of scratch device memory a launch needs for these shapes.  The caller

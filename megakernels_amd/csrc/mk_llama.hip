@@ -36,6 +36,7 @@
 // the Python VM narrows (python_vm.py:29-80,127-274).
 #include <hip/hip_runtime.h>
 
+#include <climits>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -95,8 +96,9 @@ constexpr int rows_in_flight(int wanted) { return KC <= 4 ? wanted : (wanted < 2
 // workspace layout (ints unless noted)
 // ---------------------------------------------------------------------------------------------
 struct WsLayout {
-    size_t status, shards, arrive_o, arrive_d, partial, total_bytes;
+    size_t status, shards, arrive_o, arrive_d, argmax, partial, total_bytes;
 };
+constexpr int kMaxWorkers = 1024;   // workers that can report an LM-head maximum
 
 __host__ __device__ inline WsLayout ws_layout(int L, int hid, int inter, int R) {
     WsLayout w;
@@ -106,6 +108,7 @@ __host__ __device__ inline WsLayout ws_layout(int L, int hid, int inter, int R) 
     w.shards = off;   off += (size_t)kShards * L * kHotRows * (kShardPad ? kShardPad : 1);
     w.arrive_o = off; off += hid / 16;
     w.arrive_d = off; off += hid / 16;
+    w.argmax = off;   off += 2 * (size_t)kMaxWorkers;  // per worker: value bits, index + 1 (0: nothing)
     off = (off + 3) & ~(size_t)3;
     w.partial = off;  // floats: [max(groups_o, groups_d)][hid]
     int g_o = hid / R, g_d = inter / R;
@@ -120,6 +123,7 @@ __host__ __device__ inline WsLayout ws_layout(int L, int hid, int inter, int R) 
 struct Smem {
     int abort;                      // set once, never cleared during a launch
     int last_flag;
+    int token;                      // *token_in, or -1
     long long t_launch;             // wall clock when the workgroup started
     mk_llama_args args;             // the launch arguments, read from here by every instruction
     int flags[kOutRows / 16];       // per-block "I was the last arriver" (matvec-add)
@@ -844,9 +848,21 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
             if (layer > 0 && !poll_wait(c, ticket, true, down_jobs, release)) return false;
             trace_event(c, kEvDepReady);
             if (nblk > 0) {
+                // layer 0 of a launch that was given a token reads the embedding row itself; the
+                // worker holding the first block also makes it the residual stream (every later
+                // reader of hidden_states waits, through attention, for this worker's signal)
+                const bool from_table = layer == 0 && a.token_in != nullptr;
+                const uint16_t *src = from_table ? a.embed_table + (size_t)c.sm->token * hid : a.hidden_states;
                 XVec<KC> x;
-                load_x<KC>(x, a.hidden_states, c.lane);
+                load_x<KC>(x, src, c.lane);
                 release();
+                if (from_table && start == 0) {
+#pragma unroll
+                    for (int j = 0; j < KC; j++)
+#pragma unroll
+                        for (int e = 0; e < 8; e += 2)
+                            st_u32(a.hidden_states + j * 512 + c.lane * 8 + e, mkm::pack_bf16(x.v[j][e], x.v[j][e + 1]));
+                }
                 uint4 xq[KC];
                 rms_norm_x<KC>(xq, x, wraw, a.rms_norm_eps);
                 x_to_lds<KC>(xq, c.sm, c.lane);
@@ -1131,6 +1147,20 @@ static __device__ __noinline__ bool op_matvec(SmemPtr lds, int slot, int *refusa
     return ok;
 }
 
+// (value, index) pairs: the larger value wins, the smaller index on equal values - the first maximum,
+// as torch.argmax reports it.  NaNs never win.  After the call every lane holds the wave's winner.
+__device__ __forceinline__ void argmax_combine_wave(float &v, int &i) {
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const float ov = __shfl_xor(v, off);
+        const int oi = __shfl_xor(i, off);
+        if (ov > v || (ov == v && oi < i)) {
+            v = ov;
+            i = oi;
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // opcode 7: final RMSNorm + LM head  (python_vm.py:251-274;
 // reference device op: demos/low-latency-llama/rms_lm_head.cu:10-117)
@@ -1146,6 +1176,8 @@ static __device__ __noinline__ bool op_lm_head(SmemPtr lds, int slot, int *refus
     const int down_jobs = (a.intermediate_size / a.matvec_reduction_size) * (hid / 16);
     const int blocks_per_batch = kOutRows / 16;
     const WeightBuffer W = weight_buffer(a.lm_head_weights, (size_t)a.vocab_size * hid * 2);
+    float best_v = -INFINITY;
+    int best_i = INT_MAX;
     PollTicket ticket = {nullptr, 0, 0};
     uint4 wraw[KC];
     bool first = true;
@@ -1174,13 +1206,28 @@ static __device__ __noinline__ bool op_lm_head(SmemPtr lds, int slot, int *refus
             },
             [&]() {},
             [&]() {
-                for (int p = c.lane; p < nblk * 8; p += 64)
-                    st_u32(a.logits + b0 * 16 + p * 2, mkm::pack_bf16(c.sm->out[p * 2], c.sm->out[p * 2 + 1]));
+                for (int p = c.lane; p < nblk * 8; p += 64) {
+                    const float y0 = c.sm->out[p * 2], y1 = c.sm->out[p * 2 + 1];
+                    st_u32(a.logits + b0 * 16 + p * 2, mkm::pack_bf16(y0, y1));
+                    // running maximum of this lane; rows ascend, so "greater" keeps the first maximum
+                    const int row = b0 * 16 + p * 2;
+                    if (y0 > best_v) { best_v = y0; best_i = row; }
+                    if (y1 > best_v) { best_v = y1; best_i = row + 1; }
+                }
             });
         if (!ok) return false;
         first = false;
         b0 = b1;
     } while (b0 < end);
+    if (c.controller && a.token_out) {
+        // this worker's maximum logit (the values are bf16-exact) and its first index
+        argmax_combine_wave(best_v, best_i);
+        if (c.lane == 0 && best_i != INT_MAX) {
+            int *slot_out = ws_ints(c) + ws_regions(c).argmax + 2 * (size_t)c.worker;
+            st_i32(slot_out, __builtin_bit_cast(int, best_v));
+            st_i32(slot_out + 1, best_i + 1);
+        }
+    }
     return true;
 }
 
@@ -1583,6 +1630,13 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
         sm->abort = 0;
         sm->last_flag = 0;
         sm->t_launch = wall_clock64();
+        // the token whose embedding row starts the step (written by the previous launch or the host)
+        int token = -1;
+        if (a.token_in) {
+            const long long t = *as_global(a.token_in);
+            if (t >= 0 && t < a.vocab_size) token = (int)t;
+        }
+        sm->token = token;
     }
     {
         // the launch arguments: kernarg segment -> LDS, one word per thread
@@ -1608,7 +1662,12 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
     // callee-saved register traffic (dozens of scratch stores and reloads per instruction) from
     // handlers that only this kernel calls.
     int refusal = 0;
-    for (int slot = 0; slot < a.num_slots; slot++) {
+    if (a.token_in && sm->token < 0) {
+        // every workgroup sees the same bad token and skips its queue
+        if (tid == kConsumerThreads) record_status(make_ctx(sm, 0, 0), MK_STATUS_BAD_TOKEN);
+        refusal = MK_STATUS_BAD_TOKEN;
+    }
+    for (int slot = 0; slot < a.num_slots && refusal == 0; slot++) {
         const int opcode = sm->queue[slot][0];
         if (opcode == 0) continue;  // NoOp pads the queues (megakernels/scheduler.py:287-289)
         {
@@ -1657,7 +1716,46 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
                     st_i32(p, 0);
                 }
             }
-            if (total) add_i32(a.barriers + ((size_t)(i / kHotRows) * MK_BARRIER_ROWS + 2 + i % kHotRows) * cols, total);
+            if (total && !(a.flags & MK_FLAG_RESET_BARRIERS))
+                add_i32(a.barriers + ((size_t)(i / kHotRows) * MK_BARRIER_ROWS + 2 + i % kHotRows) * cols, total);
+        }
+        if (a.flags & MK_FLAG_RESET_BARRIERS) {
+            const int words = a.num_layers * MK_BARRIER_ROWS * cols;
+            for (int i = tid; i < words; i += kThreads) st_i32(a.barriers + i, 0);
+        }
+        if (a.token_out) {
+            // the workers' LM-head maxima -> the step's token
+            int *maxima = static_cast<int *>(a.workspace) + wl.argmax;
+            float v = -INFINITY;
+            int idx = INT_MAX;
+            for (int w = tid; w < (int)gridDim.x; w += kThreads) {
+                const int stored = ld_i32(maxima + 2 * w + 1);
+                if (stored) {
+                    const float wv = __builtin_bit_cast(float, ld_i32(maxima + 2 * w));
+                    if (wv > v || (wv == v && stored - 1 < idx)) {
+                        v = wv;
+                        idx = stored - 1;
+                    }
+                    st_i32(maxima + 2 * w + 1, 0);
+                }
+            }
+            argmax_combine_wave(v, idx);
+            if (tid % 64 == 0) {
+                sm->out[2 * (tid / 64)] = v;
+                sm->flags[tid / 64] = idx;
+            }
+            wg_barrier();
+            if (tid == 0) {
+                for (int w = 1; w < kThreads / 64; w++) {
+                    const float wv = sm->out[2 * w];
+                    const int wi = sm->flags[w];
+                    if (wv > v || (wv == v && wi < idx)) {
+                        v = wv;
+                        idx = wi;
+                    }
+                }
+                *as_global(a.token_out) = idx == INT_MAX ? 0 : (long long)idx;
+            }
         }
         if (tid == 0) st_i32(&status[kDoneSlot], 0);
     }
@@ -1753,6 +1851,13 @@ int mk_llama_launch(const mk_llama_args *args, void *hip_stream) {
         return fail(-4, "pos_id %d outside the KV cache (%d) or rope table (%d)", a.pos_id, a.kv_max_len,
                     a.rope_positions);
     if (a.max_partials < 1) return fail(-3, "max_partials must be positive");
+    if (a.num_workers > kMaxWorkers) return fail(-3, "at most %d workers", kMaxWorkers);
+    if (a.token_in) {
+        if (!a.embed_table) return fail(-2, "token_in needs embed_table");
+        if ((uintptr_t)a.embed_table % 16 || (uintptr_t)a.token_in % 8)
+            return fail(-2, "embed_table must be 16-byte aligned and token_in 8-byte aligned");
+    }
+    if (a.token_out && (uintptr_t)a.token_out % 8) return fail(-2, "token_out must be 8-byte aligned");
     // weight rows are addressed as 32-bit offsets into one buffer per matrix
     const uint64_t widest = 2ull * hid * (uint64_t)(a.vocab_size > a.intermediate_size ? a.vocab_size : a.intermediate_size);
     if (widest >= (1ull << 31)) return fail(-3, "a weight matrix of %llu bytes exceeds the 2 GiB a buffer can address", (unsigned long long)widest);

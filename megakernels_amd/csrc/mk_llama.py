@@ -45,6 +45,7 @@ class MkLlamaArgs(ctypes.Structure):
             "rope_positions", "matvec_reduction_size", "attn_reduction_size")]
         + [("workspace", _P), ("workspace_bytes", ctypes.c_uint64),
            ("spin_limit_us", ctypes.c_uint32), ("flags", ctypes.c_uint32)]
+        + [("embed_table", _P), ("token_in", _P), ("token_out", _P)]
     )
 
 
@@ -98,6 +99,12 @@ def _check(t: torch.Tensor, dtype: torch.dtype, name: str) -> int:
     return t.data_ptr()
 
 
+def _token_pointer(t, name):
+    if not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype != torch.int64 or t.numel() != 1:
+        raise RuntimeError(f"{name} must be a one-element int64 device tensor")
+    return t.data_ptr()
+
+
 def mk_llama(
     barriers, instructions, timings,
     qkv_weights, attn_norm_weights, o_weights, mlp_norm_weights,
@@ -107,9 +114,18 @@ def mk_llama(
     silu_out, logits,
     pos_id, attn_scale, rms_norm_eps, skip_attn_reduction,
     stream=None,
+    *,
+    embed_table=None, token_in=None, token_out=None, reset_barriers=False,
 ):
     """Launch one decode step asynchronously on ``stream`` (a torch stream;
-    default: the current one).  Shapes are taken from the tensors."""
+    default: the current one).  Shapes are taken from the tensors.
+
+    The keyword-only arguments fold the glue of the decode loop into the
+    launch (no counterpart in the reference binding): ``token_in`` / ``token_out``
+    are one-element int64 device tensors (views into the token buffer) - the
+    step starts from ``embed_table[token_in]`` instead of ``hidden_states`` and
+    writes ``argmax(logits)`` to ``token_out``; ``reset_barriers`` leaves
+    ``barriers`` zeroed for the next launch."""
     lib = load_library()
     bf, f32, i32 = torch.bfloat16, torch.float32, torch.int32
     a = MkLlamaArgs()
@@ -185,7 +201,14 @@ def mk_llama(
     a.workspace = ws.data_ptr()
     a.workspace_bytes = ws.numel() * 4
     a.spin_limit_us = int(spin_limit_us)
-    a.flags = 1 if (record_timings and timings is not None) else 0
+    a.flags = (1 if (record_timings and timings is not None) else 0) | (2 if reset_barriers else 0)
+    if token_in is not None:
+        if embed_table is None or tuple(embed_table.shape) != (vocab, hidden):
+            raise RuntimeError("token_in needs embed_table of shape [vocab, hidden]")
+        a.embed_table = _check(embed_table, bf, "embed_table")
+        a.token_in = _token_pointer(token_in, "token_in")
+    if token_out is not None:
+        a.token_out = _token_pointer(token_out, "token_out")
 
     if stream is None:
         stream = torch.cuda.current_stream(barriers.device)
@@ -195,7 +218,8 @@ def mk_llama(
 
 
 STATUS_NAMES = {0: "ok", 1: "barrier wait timed out", 2: "unknown opcode",
-                3: "attention partition longer than the on-chip score buffer", 4: "malformed instruction"}
+                3: "attention partition longer than the on-chip score buffer", 4: "malformed instruction",
+                5: "input token outside the vocabulary"}
 
 
 def read_status(device=None, stream=None):

@@ -16,7 +16,7 @@ from megakernels_amd.demos.latency.instructions import Globals
 from megakernels_amd.mk import MK_Interpreter
 
 
-def interpret_with_mk(globs: Globals, mk_func):
+def interpret_with_mk(globs: Globals, mk_func, **fused):
     # [L, B, T, KVH, D] -> [(L B), T, KVH, D]; a view, the cache is contiguous
     k_cache_4d = globs.k_cache.flatten(0, 1)
     v_cache_4d = globs.v_cache.flatten(0, 1)
@@ -55,9 +55,18 @@ def interpret_with_mk(globs: Globals, mk_func):
         globs.rms_norm_eps,
         globs.skip_attn_reduction,
         stream=torch.cuda.current_stream(),
+        **fused,
     )
 
 
 class LatencyMK_Interpreter(MK_Interpreter):
     def interpret(self, globs: Globals):
         interpret_with_mk(globs, self.mk_func)
+
+    def interpret_step(self, globs: Globals, embed_table, token_in, token_out):
+        """One whole decode step in one launch: embedding row of ``token_in``,
+        the instruction stream, ``argmax`` into ``token_out``, barriers left
+        zeroed (no counterpart in the reference, whose loop does these around
+        the launch, ``megakernels/generators.py:121-143``)."""
+        interpret_with_mk(globs, self.mk_func, embed_table=embed_table, token_in=token_in,
+                          token_out=token_out, reset_barriers=True)

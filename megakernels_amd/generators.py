@@ -72,6 +72,7 @@ class MK_Generator(Generator):
         barrier_fill_val: int = 0,
         skip_mk: bool = False,
         skip_rest: bool = False,
+        fused_step: bool | None = None,
     ):
         self.model = model
         self.interpreter = interpreter
@@ -79,6 +80,11 @@ class MK_Generator(Generator):
         self.barrier_fill_val = barrier_fill_val
         self.skip_mk = skip_mk
         self.skip_rest = skip_rest
+        # One launch per token when the interpreter can do the embedding lookup, the barrier reset
+        # and the argmax itself; otherwise (and on request) the reference's sequence of small
+        # kernels around the launch.
+        can_fuse = hasattr(interpreter, "interpret_step") and barrier_fill_val == 0 and not skip_mk and not skip_rest
+        self.fused_step = can_fuse if fused_step is None else (fused_step and can_fuse)
         self.fill()
 
     def fill(self):
@@ -101,6 +107,15 @@ class MK_Generator(Generator):
         return torch.argmax(globs.logits, dim=-1)
 
     def generate(self, output_tokens: Tensor, prompt_len: int, ntok: int, ntok_already_generated: int = 1):
+        if self.fused_step and output_tokens.dtype == torch.int64 and output_tokens.is_contiguous():
+            globs = self.schedule.globs
+            embed = self.model.model.embed_tokens.weight
+            self.fill()
+            for i in range(ntok):
+                src = ntok_already_generated + i - 1
+                globs.pos_id = prompt_len + ntok_already_generated + i - 1
+                self.interpreter.interpret_step(globs, embed, output_tokens[0, src : src + 1], output_tokens[0, src + 1 : src + 2])
+            return
         for i in range(ntok):
             src = ntok_already_generated + i - 1
             pos_id = prompt_len + ntok_already_generated + i - 1

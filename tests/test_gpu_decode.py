@@ -21,7 +21,7 @@ def _interpreter():
     return LatencyMK_Interpreter(), sys.modules["mk_llama"]
 
 
-def _decode_case(cfg, workers, prefill, ntok, partitions=1, max_len=256, sched="rr"):
+def _decode_case(cfg, workers, prefill, ntok, partitions=1, max_len=256, sched="rr", fused=False):
     from megakernels_amd.generators import MK_Generator
     from oracle import pyvm
 
@@ -39,16 +39,52 @@ def _decode_case(cfg, workers, prefill, ntok, partitions=1, max_len=256, sched="
 
     tokens_gpu = torch.zeros(1, ntok + 1, dtype=torch.long, device="cuda:0")
     tokens_gpu[0, 0] = 5
-    MK_Generator(model_gpu, interp, schedule_gpu).generate(tokens_gpu, prompt_len=prefill, ntok=ntok)
+    gen = MK_Generator(model_gpu, interp, schedule_gpu, fused_step=fused)
+    assert gen.fused_step == fused
+    gen.generate(tokens_gpu, prompt_len=prefill, ntok=ntok)
     mk_mod.check_status("cuda:0")
     assert tokens_gpu.cpu().tolist() == tokens_cpu.tolist()
     rows = slice(prefill, prefill + ntok)
-    report = mismatches(schedule.globs, schedule_gpu.globs, kv_rows=rows)
+    names = list(schedule.globs.mutable_tensor_names())
+    if fused:
+        # one launch per token: embedding, argmax and barrier reset happen inside it, so the
+        # barriers end up zeroed instead of holding the last step's counts
+        names.remove("barriers")
+        assert int(schedule_gpu.globs.barriers.abs().sum()) == 0
+    report = mismatches(schedule.globs, schedule_gpu.globs, names=names, kv_rows=rows)
     assert not report, report
 
 
 def test_decode_tiny():
     _decode_case(config_tiny(), workers=16, prefill=20, ntok=12)
+
+
+def test_decode_tiny_one_launch_per_token():
+    _decode_case(config_tiny(), workers=16, prefill=20, ntok=12, fused=True)
+
+
+def test_decode_tiny_one_launch_per_token_split_kv():
+    _decode_case(config_tiny(), workers=16, prefill=30, ntok=20, partitions=3, fused=True)
+
+
+def test_decode_1b_slice_one_launch_per_token():
+    _decode_case(config_1b_slice(layers=3), workers=256, prefill=100, ntok=8, fused=True)
+
+
+def test_token_outside_the_vocabulary_is_reported():
+    from megakernels_amd.generators import MK_Generator
+
+    cfg = config_tiny()
+    model = make_model(cfg, max_len=64)
+    fill_kv(model, upto=8)
+    schedule = build_schedule(model, 16)
+    model_gpu, schedule_gpu = mirror_to_gpu(model, schedule)
+    interp, mk_mod = _interpreter()
+    tokens = torch.zeros(1, 3, dtype=torch.long, device="cuda:0")
+    tokens[0, 0] = cfg.vocab_size + 7
+    MK_Generator(model_gpu, interp, schedule_gpu, fused_step=True).generate(tokens, prompt_len=8, ntok=1)
+    code, *_ = mk_mod.read_status("cuda:0")
+    assert code == 5
 
 
 def test_decode_tiny_split_kv_crossing_block_boundaries():
