@@ -90,6 +90,9 @@ constexpr int kDoneSlot = 8;        // workspace int: workgroups finished
 template <int KC>
 constexpr int rows_in_flight(int wanted) { return KC <= 4 ? wanted : (wanted < 2 ? wanted : 2); }
 
+#ifndef MK_POLL_SLEEP
+#define MK_POLL_SLEEP 10            // units of 64 clocks between two looks at a dependency
+#endif
 #define AG __HIP_MEMORY_SCOPE_AGENT
 
 // ---------------------------------------------------------------------------------------------
@@ -469,7 +472,9 @@ __device__ __forceinline__ bool poll_wait(const Ctx &c, PollTicket t, bool sum_m
             if (c.lane == 0) record_status(c, MK_STATUS_BARRIER_TIMEOUT);
             return false;
         }
-        __builtin_amdgcn_s_sleep(1);
+        // a quarter microsecond between looks: more looks (or two in flight) only add traffic on
+        // the counters' memory channels and make the step slower
+        __builtin_amdgcn_s_sleep(MK_POLL_SLEEP);
         v = t.ptr ? ld_i32(t.ptr) : 0;
         st = c.lane == 63 ? ld_i32(status) : 0;
     }
