@@ -90,6 +90,9 @@ constexpr int kDoneSlot = 8;        // workspace int: workgroups finished
 template <int KC>
 constexpr int rows_in_flight(int wanted) { return KC <= 4 ? wanted : (wanted < 2 ? wanted : 2); }
 
+#ifndef MK_PAIR_OPROJ_UPGATE
+#define MK_PAIR_OPROJ_UPGATE 1      // O-proj and a directly following up/gate run as one handler
+#endif
 #ifndef MK_POLL_SLEEP
 #define MK_POLL_SLEEP 10            // units of 64 clocks between two looks at a dependency
 #endif
@@ -1152,6 +1155,50 @@ static __device__ __noinline__ bool op_matvec(SmemPtr lds, int slot, int *refusa
     return ok;
 }
 
+// O-proj followed directly by up/gate, as one handler.  O-proj is short (two rows per wave in the
+// usual schedule) and waits long (for attention); the worker that runs it would otherwise request its
+// up/gate rows only after O-proj's epilogue, when up/gate's dependency is about to resolve - half of
+// the workers would fetch all of their up/gate rows on the critical path.  Here the first up/gate rows
+// are requested together with the O-proj rows, and the two O-proj buffers go to up/gate as soon as
+// O-proj is done.  Returns the number of instructions executed (2, or 1 when the second instruction
+// is malformed and left to report itself), 0 on failure.
+template <int KC>
+static __device__ __noinline__ int op_oproj_upgate(SmemPtr lds, int slot, int *refusal) {
+    constexpr int NBUF = 6;
+    typedef BufMap<0, 1> MapO;
+    typedef BufMap<2, 3, 4, 5> MapU0;        // requested on entry
+    typedef BufMap<0, 1> MapU1;              // requested when O-proj is done
+    typedef BufMap<2, 3, 4, 5, 0, 1> MapU;
+    const Ctx co = make_ctx(lds, slot, 4);
+    const Ctx cu = make_ctx(lds, slot + 1, 5);
+    MatvecDesc dso, dsu;
+    if (!describe_matvec(lds, slot, dso)) {
+        bail(co, MK_STATUS_BAD_INSTRUCTION, refusal);
+        return 0;
+    }
+    const bool pair = describe_matvec(lds, slot + 1, dsu);
+    if (co.controller) {
+        if (!control_matvec<KC>(co)) return 0;
+        if (!pair) return 1;
+        trace_event(co, kEvEnd);
+        trace_event(cu, kEvStart);
+        if (cu.trace && cu.lane == 0) st_plain_i32(cu.trace + kEvOpcode, 5);
+        return control_matvec<KC>(cu) ? 2 : 0;
+    }
+    if (!pair) dsu = dso;  // never fetched: the requests below become no-ops
+    const int mine_o = rows_of_wave(dso.ntasks, co.wave);
+    const int mine_u = pair ? rows_of_wave(dsu.ntasks, co.wave) : 0;
+    uint4 pool[NBUF][KC];
+    wg_barrier();  // entry of O-proj: the controller's first requests are out
+    request_rows<KC, MapO>(co, pool, dso, 0, mine_o);
+    request_rows<KC, MapU0>(co, pool, dsu, 0, mine_u, pair);
+    if (!consumer_run<KC, MapO>(co, pool, dso, mine_o)) return 0;
+    request_rows<KC, MapU1>(co, pool, dsu, MapU0::size, mine_u, pair);
+    if (!pair) return 1;
+    wg_barrier();  // entry of up/gate: its first requests went out long ago
+    return consumer_run<KC, MapU>(cu, pool, dsu, mine_u) ? 2 : 0;
+}
+
 // (value, index) pairs: the larger value wins, the smaller index on equal values - the first maximum,
 // as torch.argmax reports it.  NaNs never win.  After the call every lane holds the wave's winner.
 __device__ __forceinline__ void argmax_combine_wave(float &v, int &i) {
@@ -1685,14 +1732,24 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
         case 1: ok = op_matvec<1, KC_HID>(sm, slot, &refusal); break;
         case 2: ok = op_attention<D>(sm, slot, &refusal); break;
         case 3: ok = op_attention_reduction<D>(sm, slot, &refusal); break;
-        case 4: ok = op_matvec<4, KC_RED>(sm, slot, &refusal); break;
+        case 4:
+            if constexpr (KC_HID == KC_RED && MK_PAIR_OPROJ_UPGATE) {
+                if (slot + 1 < a.num_slots && sm->queue[slot + 1][0] == 5) {
+                    const int executed = op_oproj_upgate<KC_HID>(sm, slot, &refusal);
+                    ok = executed > 0;
+                    slot += ok ? executed - 1 : 0;
+                    break;
+                }
+            }
+            ok = op_matvec<4, KC_RED>(sm, slot, &refusal);
+            break;
         case 5: ok = op_matvec<5, KC_HID>(sm, slot, &refusal); break;
         case 6: ok = op_matvec<6, KC_RED>(sm, slot, &refusal); break;
         case 7: ok = op_lm_head<KC_HID>(sm, slot, &refusal); break;
         default: ok = bail(make_ctx(sm, slot, opcode), MK_STATUS_BAD_OPCODE, &refusal);  // reference: trap, include/util.cuh:38
         }
         if (!ok) break;
-        trace_event(make_ctx(sm, slot, opcode), kEvEnd);
+        trace_event(make_ctx(sm, slot, sm->queue[slot][0]), kEvEnd);
     }
     if (refusal && tid == 0) sm->abort = refusal;
 
