@@ -70,8 +70,11 @@ constexpr int kDoneSlot = 8;        // workspace int: workgroups finished
 
 // Weight rows in flight per consumer wave, per instruction kind (16 VGPRs per 2048-element row; the
 // 9-wave workgroup leaves each lane 168 VGPRs).  The rows requested before the dependency wait are
-// the prefetch; rows a wave does not have become no-op requests, so the depth follows the rows per
-// wave of the usual schedules: QKV 2, O-proj 1, up/gate 8, down 4.
+// the prefetch; rows a wave does not have become no-op requests.  Rows per wave in the usual
+// schedules: QKV 2, O-proj 2, up/gate 8, down 4, LM head 63.  The depths come from sweeps of the
+// whole decode step: an instruction that everybody enters at the same moment, right after its
+// dependency resolves (down, LM head), does best with a shallow queue - deep ones only delay the
+// first rows - while up/gate, entered early, takes all the rows the registers hold.
 #ifndef MK_PF_QKV
 #define MK_PF_QKV 2
 #endif
@@ -82,10 +85,10 @@ constexpr int kDoneSlot = 8;        // workspace int: workgroups finished
 #define MK_PF_UPGATE 5
 #endif
 #ifndef MK_PF_DOWN
-#define MK_PF_DOWN 3
+#define MK_PF_DOWN 2
 #endif
 #ifndef MK_PF_LMHEAD
-#define MK_PF_LMHEAD 4
+#define MK_PF_LMHEAD 2
 #endif
 template <int KC>
 constexpr int rows_in_flight(int wanted) { return KC <= 4 ? wanted : (wanted < 2 ? wanted : 2); }
