@@ -1,0 +1,111 @@
+"""Per-instruction timeline of one decode step, from the megakernel's own timing records.
+
+    python -m megakernels_amd.scripts.timeline [layers=16] [pos=4100] [partitions=0] [layer=1]
+
+Builds the random-initialised 1B architecture with ``layers`` layers, fills the KV cache up to ``pos``
+with seeded noise, runs a few warm-up steps, then one step with ``MK_FLAG_TIMINGS`` set and prints,
+per instruction kind, how long the workers waited for the dependency, loaded the activation vector,
+computed and wrote back; and for one layer when each kind started, saw its dependency and ended across
+the workers.  The reference records the same events (``include/util.cuh:215-246``) when compiled with
+``TIMING_RECORD_ENABLED``; here the records are taken on request at run time.
+
+Times are microseconds since the workgroup started (100 MHz wall clock of the device).
+"""
+
+from __future__ import annotations
+
+import sys
+
+import numpy as np
+import torch
+
+from megakernels_amd.demos.latency.scheduler import LatencyScheduleBuilder, pick_num_attention_partitions
+from megakernels_amd.dispatch import make_mk_interpreter
+from megakernels_amd.llama import LlamaConfig, LlamaForCausalLM
+from megakernels_amd.model_types import ExtraModelConfig
+from megakernels_amd.scheduler import assign_to_sms, tensorize_instructions
+from megakernels_amd.utils import get_sm_count, set_sm_count_override
+
+NAMES = {1: "qkv", 2: "attention", 3: "merge", 4: "o-proj", 5: "up/gate", 6: "down", 7: "lm-head"}
+
+
+def main(argv):
+    opts = {"layers": 16, "pos": 4100, "partitions": 0, "layer": 1, "sched": "rr"}
+    for arg in argv:
+        key, _, value = arg.partition("=")
+        if key not in opts:
+            raise SystemExit(f"unknown option {key}; known: {', '.join(opts)}")
+        opts[key] = value if key == "sched" else int(value)
+    if not torch.cuda.is_available():
+        raise SystemExit("timeline needs a GPU")
+    device = torch.device("cuda:0")
+    cfg = LlamaConfig.llama_1b()
+    cfg.num_hidden_layers = opts["layers"]
+    pos = opts["pos"]
+    model = LlamaForCausalLM.from_random(cfg, ExtraModelConfig(interleave_rope=True, max_len_override=pos + 64), seed=0)
+    gen = torch.Generator().manual_seed(2)
+    for cache in model.stacked_kv_cache:
+        shape = list(cache.shape)
+        shape[2] = pos
+        cache[:, :, :pos] = torch.randn(shape, generator=gen).to(cache.dtype)
+    model = model.to(device)
+    workers = get_sm_count(device)
+    set_sm_count_override(workers)
+    partitions = opts["partitions"] or pick_num_attention_partitions(pos, 1)
+    schedule = LatencyScheduleBuilder.build(model, num_attention_partitions=partitions)
+    tensorize_instructions(schedule.globs, assign_to_sms(opts["sched"], schedule=schedule))
+    globs = schedule.globs
+    interpreter = make_mk_interpreter("latency")
+    mk = sys.modules["mk_llama"]
+    globs.hidden_states.copy_(model.model.embed_tokens.weight[5])
+    globs.pos_id = pos
+    for _ in range(3):
+        globs.barriers.zero_()
+        interpreter.interpret(globs)
+    mk.check_status(device)
+    mk.record_timings = True
+    globs.barriers.zero_()
+    globs.timings.zero_()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    interpreter.interpret(globs)
+    end.record()
+    torch.cuda.synchronize()
+    mk.record_timings = False
+    mk.check_status(device)
+
+    # [workers, slots, 6]: start, dependency seen, activation ready, rows done, end, opcode
+    t = globs.timings.cpu()[:, :, :6].numpy().astype(np.float64)
+    ins = globs.instructions.cpu().numpy()
+    t[:, :, :5] /= 100.0
+    print(f"{opts['layers']} layers, position {pos}, {partitions} attention partitions, {workers} workers, "
+          f"assignment {opts['sched']}: kernel {start.elapsed_time(end) * 1e3:.1f} us with timing records on, "
+          f"last instruction ends at {t[:, :, 4].max():.1f} us")
+    print("\nper instruction kind, mean / max over all instructions (us):")
+    print(f"{'kind':10s} {'count':>6s} {'wait for dependency':>20s} {'activation':>14s} {'rows':>14s} {'write back':>14s}")
+    for op, name in NAMES.items():
+        sel = t[:, :, 5] == op
+        if not sel.any():
+            continue
+        st, dep, inp, rows, done = (t[:, :, i][sel] for i in range(5))
+        if op in (2, 3):
+            inp = dep  # these record no separate activation event
+        cell = lambda a: f"{a.mean():6.2f} /{a.max():6.2f}"
+        print(f"{name:10s} {int(sel.sum()):6d} {cell(dep - st):>20s} {cell(inp - dep):>14s} {cell(rows - inp):>14s} {cell(done - rows):>14s}")
+    layer = min(opts["layer"], opts["layers"] - 1)
+    print(f"\nlayer {layer}, over the workers that run the kind (us): first start | dependency seen p10 p50 max | end p10 p50 max")
+    for op in range(1, 7):
+        sel = (ins[:, :, 0] == op) & (ins[:, :, 1] == layer)
+        if not sel.any():
+            continue
+        st, dep, done = t[:, :, 0][sel], t[:, :, 1][sel], t[:, :, 4][sel]
+        q = lambda a, ps: " ".join(f"{np.percentile(a, p):7.2f}" for p in ps)
+        print(f"  {NAMES[op]:10s} {st.min():7.2f} | {q(dep, (10, 50, 100))} | {q(done, (10, 50, 100))}")
+    sel = ins[:, :, 0] == 7
+    if sel.any():
+        print(f"  {'lm-head':10s} {t[:, :, 0][sel].min():7.2f} | {np.percentile(t[:, :, 1][sel], 50):7.2f} (p50) | "
+              f"{t[:, :, 4][sel].max():7.2f} (max)")
+
+
+if __name__ == "__main__":
+    main(sys.argv[1:])
