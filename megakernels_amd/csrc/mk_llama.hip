@@ -5,16 +5,18 @@
 //   * grid = one workgroup per compute unit; workgroup w executes instructions[w, 0..num_slots)
 //     strictly in order.  The LDS request (> half of the CU's 160 KB) keeps a second workgroup
 //     off the same CU.
-//   * a workgroup is 9 wave64: eight CONSUMER waves stream weight rows (16-byte global loads
-//     straight into VGPRs, several rows in flight per wave, no LDS staging for weights) and do
-//     the dot products; one CONTROLLER wave does everything that is latency-critical and small:
+//   * a workgroup is 9 wave64: eight CONSUMER waves stream weight rows (16-byte streaming buffer
+//     loads straight into VGPRs, several rows in flight per wave, no LDS staging for weights) and
+//     do the dot products; one CONTROLLER wave does everything that is latency-critical and small:
 //     it waits on the dependency counters, fetches the activation vector, normalises it and hands
 //     it to the consumers through LDS, and after the matvec it runs the epilogue (RoPE, SiLU,
 //     residual, stores) and signals the next counter.  The controller never has bulk loads
 //     outstanding, so its polls and 4 KB activation loads do not queue behind its own weight
-//     traffic (vector memory returns in order per wave).  Consumers request the first rows of the
-//     NEXT instruction as soon as they finish the current one, before any dependency is checked:
-//     weights never depend on a barrier.
+//     traffic (vector memory returns in order per wave).  Consumers request the first rows of an
+//     instruction on entry, before its dependency is known: weights never depend on a barrier.
+//     (In attention and in the partition merge the consumer waves also store and signal.)
+//   * launch arguments and the worker's instruction queue are copied into LDS once; every
+//     instruction kind has its own non-inlined handler, so each gets its own register allocation.
 //   * cross-CU ordering is only through counters in HBM, with the counts of the reference's
 //     Python VM (megakernels/demos/latency/python_vm.py).  The eight XCDs have private L2
 //     caches, so everything one CU writes for another (activations, the new KV row, counters)
@@ -666,12 +668,7 @@ __device__ __forceinline__ bool controller_sequence(const Ctx &c, Ahead ahead, P
     // after the controller has requested the activation vector.  A worker that arrives late then
     // has its short critical requests ahead of its own prefetch instead of behind it.
     ahead();
-#ifdef MK_NO_GATE
-    bool released = true;
-    wg_barrier();
-#else
     bool released = false;
-#endif
     auto release = [&]() {
         if (!released) wg_barrier();
         released = true;
