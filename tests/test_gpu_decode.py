@@ -71,6 +71,12 @@ def test_decode_1b_slice_one_launch_per_token():
     _decode_case(config_1b_slice(layers=3), workers=256, prefill=100, ntok=8, fused=True)
 
 
+def test_decode_1b_slice_many_steps_split_kv_one_launch_per_token():
+    # 160 consecutive launches, every one checked through its token: a race between workgroups would
+    # have many chances to show
+    _decode_case(config_1b_slice(layers=2), workers=256, prefill=500, ntok=160, partitions=3, max_len=1024, fused=True)
+
+
 def test_token_outside_the_vocabulary_is_reported():
     from megakernels_amd.generators import MK_Generator
 
