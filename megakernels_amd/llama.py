@@ -93,8 +93,19 @@ class LlamaConfig:
 
         raw = json.loads(Path(path).read_text())
         known = {k: raw[k] for k in cls.__dataclass_fields__ if k in raw}
-        if "head_dim" not in known:
+        if known.get("head_dim") is None:
             known["head_dim"] = raw["hidden_size"] // raw["num_attention_heads"]
+        # transformers 4.x writes `rope_theta` and `rope_scaling`; 5.x writes one `rope_parameters`
+        # dict holding the base as well.  A checkpoint without scaling has none: say so explicitly,
+        # the dataclass default is the Llama-3.2 scaling.
+        params = raw.get("rope_parameters")
+        if params:
+            params = dict(params)
+            if "rope_theta" in params:
+                known["rope_theta"] = float(params.pop("rope_theta"))
+            known["rope_scaling"] = params
+        elif "rope_scaling" not in raw:
+            known["rope_scaling"] = None
         return cls(**known)
 
 

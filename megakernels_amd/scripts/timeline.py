@@ -1,12 +1,14 @@
 """Per-instruction timeline of one decode step, from the megakernel's own timing records.
 
-    python -m megakernels_amd.scripts.timeline [layers=16] [pos=4100] [partitions=0] [layer=1]
+    python -m megakernels_amd.scripts.timeline [layers=16] [pos=4100] [partitions=0] [layer=1] [out=trace.npz]
 
 Builds the random-initialised 1B architecture with ``layers`` layers, fills the KV cache up to ``pos``
 with seeded noise, runs a few warm-up steps, then one step with ``MK_FLAG_TIMINGS`` set and prints,
 per instruction kind, how long the workers waited for the dependency, loaded the activation vector,
 computed and wrote back; and for one layer when each kind started, saw its dependency and ended across
-the workers.  The reference records the same events (``include/util.cuh:215-246``) when compiled with
+the workers.  ``out=`` saves the raw records (``timings`` [workers, slots, 128] and ``instructions``
+[workers, slots, 32], plain ``numpy`` arrays) for a Gantt view elsewhere - the counterpart of the
+reference's ``diff_test.py outfile=`` dump (``scripts/diff_test.py:231-242``).  The reference records the same events (``include/util.cuh:215-246``) when compiled with
 ``TIMING_RECORD_ENABLED``; here the records are taken on request at run time.
 
 Times are microseconds since the workgroup started (100 MHz wall clock of the device).
@@ -30,12 +32,12 @@ NAMES = {1: "qkv", 2: "attention", 3: "merge", 4: "o-proj", 5: "up/gate", 6: "do
 
 
 def main(argv):
-    opts = {"layers": 16, "pos": 4100, "partitions": 0, "layer": 1, "sched": "rr"}
+    opts = {"layers": 16, "pos": 4100, "partitions": 0, "layer": 1, "sched": "rr", "out": ""}
     for arg in argv:
         key, _, value = arg.partition("=")
         if key not in opts:
             raise SystemExit(f"unknown option {key}; known: {', '.join(opts)}")
-        opts[key] = value if key == "sched" else int(value)
+        opts[key] = value if key in ("sched", "out") else int(value)
     if not torch.cuda.is_available():
         raise SystemExit("timeline needs a GPU")
     device = torch.device("cuda:0")
@@ -78,6 +80,9 @@ def main(argv):
     t = globs.timings.cpu()[:, :, :6].numpy().astype(np.float64)
     ins = globs.instructions.cpu().numpy()
     t[:, :, :5] /= 100.0
+    if opts["out"]:
+        np.savez_compressed(opts["out"], timings=globs.timings.cpu().numpy(), instructions=ins,
+                            ticks_per_microsecond=np.array(100))
     print(f"{opts['layers']} layers, position {pos}, {partitions} attention partitions, {workers} workers, "
           f"assignment {opts['sched']}: kernel {start.elapsed_time(end) * 1e3:.1f} us with timing records on, "
           f"last instruction ends at {t[:, :, 4].max():.1f} us")

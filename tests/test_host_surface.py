@@ -215,3 +215,38 @@ def test_shim_refuses_cpu_tensors_and_missing_library(monkeypatch):
     monkeypatch.setattr(mod, "LIBRARY", mod.LIBRARY.with_name("missing.so"))
     with pytest.raises(RuntimeError, match="missing"):
         mod.load_library()
+
+
+def test_from_pretrained_reads_a_hugging_face_checkpoint_and_matches_its_forward(tmp_path):
+    """A checkpoint directory written by the installed third-party `transformers` (random tiny Llama with
+    llama3 rope scaling, untied head) is loaded by `from_pretrained`; both the interleaved and the
+    half-split model must reproduce the third-party model's logits.  Pins the name mapping, the
+    rotary-pair row permutation and the PyTorch forward against an independent implementation."""
+    transformers = pytest.importorskip("transformers")
+    hf_cfg = transformers.LlamaConfig(
+        vocab_size=512, hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+        num_key_value_heads=2, head_dim=64, max_position_embeddings=256, rms_norm_eps=1e-5, rope_theta=500000.0,
+        tie_word_embeddings=False, attention_bias=False, mlp_bias=False,
+        rope_scaling={"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                      "original_max_position_embeddings": 64},
+    )
+    torch.manual_seed(11)
+    hf = transformers.LlamaForCausalLM(hf_cfg).to(torch.float32).eval()
+    hf.save_pretrained(tmp_path, safe_serialization=True)
+    ids = torch.randint(0, 512, (1, 12), generator=torch.Generator().manual_seed(5))
+    with torch.no_grad():
+        want = hf(input_ids=ids).logits[0].float()
+
+    for interleave in (True, False):
+        ours = LlamaForCausalLM.from_pretrained(
+            tmp_path, ExtraModelConfig(interleave_rope=interleave, max_len_override=32), dtype=torch.float32)
+        assert ours.config.num_hidden_layers == 2 and ours.lm_head.lm_head.weight is not ours.model.embed_tokens.weight
+        out = ours(BatchState(input_ids=ids, position_ids=torch.arange(12)))
+        logits = ours.lm_head.lm_head.weight.float() @ _final_norm(ours, out.hidden_states[0].float()).T
+        assert (logits.T - want).abs().max() <= 2e-4 * want.abs().max(), interleave
+        assert out.output_ids[0].tolist() == want.argmax(-1).tolist()
+
+
+def _final_norm(model, hidden):
+    w = model.lm_head.input_norm.weight.float()
+    return w * hidden * torch.rsqrt(hidden.pow(2).mean(-1, keepdim=True) + model.config.rms_norm_eps)
