@@ -175,6 +175,27 @@ def test_unsatisfiable_dependency_times_out_and_reports():
     test_decode_tiny()
 
 
+def test_missing_attention_partials_time_out_in_the_merge():
+    """Split-KV schedule without its attention instructions: the merging waves poll tagged values that
+    never arrive, give up at the spin limit and the whole grid drains."""
+    model = make_model(config_tiny())
+    fill_kv(model, upto=40)
+    schedule = build_schedule(model, 16, partitions=2)
+    g = schedule.globs
+    g.pos_id = 40
+    g.instructions[g.instructions[:, :, 0] == 2] = 0
+    _, schedule_gpu = mirror_to_gpu(model, schedule)
+    interp, mk_mod = _interpreter()
+    mk_mod.spin_limit_us = 20000
+    try:
+        interp.interpret(schedule_gpu.globs)
+        code, worker, slot, opcode = mk_mod.read_status("cuda:0")
+    finally:
+        mk_mod.spin_limit_us = 0
+    assert code == 1 and opcode in (3, 4)
+    test_decode_tiny_split_kv_crossing_block_boundaries()
+
+
 def test_unknown_opcode_and_bad_fields_are_reported():
     model = make_model(config_tiny())
     schedule = build_schedule(model, 16)
