@@ -844,6 +844,10 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
     const int hid = a.hidden_size, D = a.head_dim, H = a.num_attention_heads, KVH = a.num_kv_heads;
     const int nblk = end > start ? end - start : 0;
     const int down_jobs = (a.intermediate_size / a.matvec_reduction_size) * (hid / 16);
+    const int k_start = H * D, v_start = k_start + KVH * D;
+    constexpr int kPre = 2;
+    float rot[kPre][4] = {{1.0f, 1.0f, 0.0f, 0.0f}, {1.0f, 1.0f, 0.0f, 0.0f}};
+    const bool prefetched = nblk * 8 <= kPre * 64;
     PollTicket ticket = {nullptr, 0, 0};
     uint4 wraw[KC];
     return controller_sequence(
@@ -877,22 +881,37 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
             }
             return true;
         },
-        [&]() {},
+        [&]() {
+            // the rotary factors of this lane's row pairs do not depend on the matvec: fetch them while
+            // the consumers work
+            if (prefetched) {
+#pragma unroll
+                for (int k = 0; k < kPre; k++) {
+                    const int p = c.lane + k * 64;
+                    const int row0 = start * 16 + p * 2;
+                    if (p < nblk * 8 && row0 < v_start) {
+                        const int d = row0 % D;
+                        const float *cs = a.rope_cos + (size_t)a.pos_id * D + d;
+                        const float *sn = a.rope_sin + (size_t)a.pos_id * D + d;
+                        rot[k][0] = ld_const_f32(cs);
+                        rot[k][1] = ld_const_f32(cs + 1);
+                        rot[k][2] = ld_const_f32(sn);
+                        rot[k][3] = ld_const_f32(sn + 1);
+                    }
+                }
+            }
+        },
         [&]() {
             // epilogue: one lane per adjacent row pair
-            const int k_start = H * D, v_start = k_start + KVH * D;
             const size_t kv_row = ((size_t)layer * a.kv_max_len + a.pos_id) * KVH * D;
-            for (int p = c.lane; p < nblk * 8; p += 64) {
+            auto emit = [&](int p, float c0, float c1, float s0, float s1) {
                 const int row0 = start * 16 + p * 2;
                 const float y0 = c.sm->out[p * 2], y1 = c.sm->out[p * 2 + 1];
                 uint32_t packed;
                 if (row0 < v_start) {
                     // interleaved rotary embedding (llama.py:136-174): products and sum in fp32, unfused
-                    const int d = row0 % D;
-                    const float *cs = a.rope_cos + (size_t)a.pos_id * D + d;
-                    const float *sn = a.rope_sin + (size_t)a.pos_id * D + d;
-                    const float even = (y0 * ld_const_f32(cs)) + ((-y1) * ld_const_f32(sn));
-                    const float odd = (y1 * ld_const_f32(cs + 1)) + (y0 * ld_const_f32(sn + 1));
+                    const float even = (y0 * c0) + ((-y1) * s0);
+                    const float odd = (y1 * c1) + (y0 * s1);
                     packed = mkm::pack_bf16(even, odd);
                 } else {
                     packed = mkm::pack_bf16(y0, y1);
@@ -902,6 +921,23 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
                 else if (row0 < v_start) dst = a.k_cache + kv_row + (row0 - k_start);
                 else dst = a.v_cache + kv_row + (row0 - v_start);
                 st_u32(dst, packed);
+            };
+            if (prefetched) {
+#pragma unroll
+                for (int k = 0; k < kPre; k++)
+                    if (c.lane + k * 64 < nblk * 8) emit(c.lane + k * 64, rot[k][0], rot[k][1], rot[k][2], rot[k][3]);
+            } else {
+                for (int p = c.lane; p < nblk * 8; p += 64) {
+                    const int row0 = start * 16 + p * 2;
+                    float c0 = 1.0f, c1 = 1.0f, s0 = 0.0f, s1 = 0.0f;
+                    if (row0 < v_start) {
+                        const int d = row0 % D;
+                        const float *cs = a.rope_cos + (size_t)a.pos_id * D + d;
+                        const float *sn = a.rope_sin + (size_t)a.pos_id * D + d;
+                        c0 = ld_const_f32(cs); c1 = ld_const_f32(cs + 1); s0 = ld_const_f32(sn); s1 = ld_const_f32(sn + 1);
+                    }
+                    emit(p, c0, c1, s0, s1);
+                }
             }
             wait_stores();
             // one arrival per block on its head's counter (python_vm.py:248)
