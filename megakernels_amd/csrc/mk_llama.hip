@@ -1801,40 +1801,57 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
     }
     wg_barrier();
     if (sm->last_flag) {
+        // One thread per (counter, shard), two pairs per trip with both loads in flight, and the
+        // workers' maxima requested before the fold: the step's token waits for one round trip here,
+        // not for a chain of them.
         const int counters = a.num_layers * kHotRows;
         int *shards = static_cast<int *>(a.workspace) + wl.shards;
         const int cols = a.num_attention_heads + 2 * a.num_kv_heads;
-        for (int i = tid; i < counters; i += kThreads) {
-            int total = 0;
-            for (int s = 0; s < kShards; s++) {
-                int *p = kShardPad ? shards + ((size_t)i * kShards + s) * kShardPad : shards + (size_t)s * counters + i;
-                const int v = ld_i32(p);
-                if (v) {
-                    total += v;
-                    st_i32(p, 0);
-                }
-            }
-            if (total && !(a.flags & MK_FLAG_RESET_BARRIERS))
-                add_i32(a.barriers + ((size_t)(i / kHotRows) * MK_BARRIER_ROWS + 2 + i % kHotRows) * cols, total);
+        const bool reset = (a.flags & MK_FLAG_RESET_BARRIERS) != 0;
+        int *maxima = static_cast<int *>(a.workspace) + wl.argmax;
+        constexpr int kMaxTrips = (kMaxWorkers + kThreads - 1) / kThreads;
+        uint64_t reported[kMaxTrips];
+#pragma unroll
+        for (int k = 0; k < kMaxTrips; k++) {
+            const int w = tid + k * kThreads;
+            reported[k] = a.token_out && w < (int)gridDim.x ? ld_u64(maxima + 2 * w) : 0;
         }
-        if (a.flags & MK_FLAG_RESET_BARRIERS) {
+        auto shard_at = [&](int k) {
+            const int i = k / kShards, sh = k % kShards;
+            return kShardPad ? shards + ((size_t)i * kShards + sh) * kShardPad : shards + (size_t)sh * counters + i;
+        };
+        auto fold = [&](int k, int v) {
+            if (v == 0) return;
+            st_i32(shard_at(k), 0);
+            const int i = k / kShards;
+            if (!reset) add_i32(a.barriers + ((size_t)(i / kHotRows) * MK_BARRIER_ROWS + 2 + i % kHotRows) * cols, v);
+        };
+        const int pairs = counters * kShards;
+        for (int k = tid; k < pairs; k += 2 * kThreads) {
+            const int k2 = k + kThreads;
+            const int v = ld_i32(shard_at(k));
+            const int v2 = k2 < pairs ? ld_i32(shard_at(k2)) : 0;
+            fold(k, v);
+            if (k2 < pairs) fold(k2, v2);
+        }
+        if (reset) {
             const int words = a.num_layers * MK_BARRIER_ROWS * cols;
             for (int i = tid; i < words; i += kThreads) st_i32(a.barriers + i, 0);
         }
         if (a.token_out) {
             // the workers' LM-head maxima -> the step's token
-            int *maxima = static_cast<int *>(a.workspace) + wl.argmax;
             float v = -INFINITY;
             int idx = INT_MAX;
-            for (int w = tid; w < (int)gridDim.x; w += kThreads) {
-                const int stored = ld_i32(maxima + 2 * w + 1);
+#pragma unroll
+            for (int k = 0; k < kMaxTrips; k++) {
+                const int stored = (int)(reported[k] >> 32);
                 if (stored) {
-                    const float wv = __builtin_bit_cast(float, ld_i32(maxima + 2 * w));
+                    const float wv = __builtin_bit_cast(float, (int)(uint32_t)reported[k]);
                     if (wv > v || (wv == v && stored - 1 < idx)) {
                         v = wv;
                         idx = stored - 1;
                     }
-                    st_i32(maxima + 2 * w + 1, 0);
+                    st_i32(maxima + 2 * (tid + k * kThreads) + 1, 0);
                 }
             }
             argmax_combine_wave(v, idx);
@@ -1968,6 +1985,7 @@ int mk_llama_launch(const mk_llama_args *args, void *hip_stream) {
     if (a.workspace_bytes < need)
         return fail(-6, "workspace has %llu bytes, %llu needed", (unsigned long long)a.workspace_bytes,
                     (unsigned long long)need);
+    if ((uintptr_t)a.workspace % 16) return fail(-6, "workspace must be 16-byte aligned");
 
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
