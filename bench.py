@@ -5,10 +5,12 @@
 One "step" is one decode step (one token): embedding row -> hidden state,
 barrier reset, the instruction stream, argmax over the logits, token write -
 the per-token loop of the reference's mk generator
-(megakernels/generators.py:121-163).  By default all of it is ONE megakernel
-launch (--loop fused); --loop reference runs the reference's sequence of small
-kernels around the launch instead.  Weights, KV cache and instruction
-tensor are resident in HBM before the timed region starts.
+(megakernels/generators.py:121-163).  By default all of it happens inside the
+megakernel, and one launch covers --launch-steps consecutive steps (--loop
+fused); --launch-steps 1 is one launch per token, and --loop reference runs the
+reference's sequence of small kernels around a launch per token instead.
+Weights, KV cache and instruction tensor are resident in HBM before the timed
+region starts.
 
 Workloads (all Llama-3.2-1B architecture, random bf16 weights N(0, 0.02) from
 seed 0, RMSNorm weights 1):
@@ -17,8 +19,9 @@ seed 0, RMSNorm weights 1):
   c3  KV cache pre-filled to 16384 positions
 
 Prints one JSON line.  `roofline` prices the megakernel alone: algorithmic
-bytes per launch (weights + norm weights + K/V read) divided by the mean
-kernel time measured with events on the launch stream.  `cpu_baseline` is the
+bytes per launch (weights + norm weights + K/V read, summed over the steps of
+the launch) divided by the mean launch duration measured with events on the
+launch stream.  `cpu_baseline` is the
 C restatement of the reference's Python VM (the parity checker) timed on this
 host's cores over a bounded number of the same decode steps; its tokens are
 also compared with the GPU's.
@@ -65,6 +68,9 @@ def main():
                     help="fused: one launch per token (embedding row, barrier reset and argmax inside the "
                          "megakernel); reference: the reference generator's sequence of small kernels around "
                          "the launch")
+    ap.add_argument("--launch-steps", type=int, default=8,
+                    help="--loop fused: decode steps per megakernel launch (the token of one step starts the "
+                         "next inside the kernel); 1 = one launch per token, 0 = all steps of a phase in one launch")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="after the timed region also run a plain 1 GiB device copy three times, so that a "
                          "rocprofv3 --pmc run of this command holds a kernel of known traffic to scale "
@@ -123,7 +129,8 @@ def main():
     schedule = LatencyScheduleBuilder.build(model, num_attention_partitions=partitions)
     tensorize_instructions(schedule.globs, assign_to_sms(args.sched, schedule=schedule))
     interpreter = make_mk_interpreter("latency")
-    gen = MK_Generator(model, interpreter, schedule, fused_step=args.loop == "fused")
+    gen = MK_Generator(model, interpreter, schedule, fused_step=args.loop == "fused",
+                       steps_per_launch=args.launch_steps if args.loop == "fused" else 1)
     mk_mod = sys.modules["mk_llama"]
 
     ntok = total_steps + 1
@@ -142,32 +149,47 @@ def main():
     # kernel-only events: wrap the interpreter so each launch is bracketed on the launch stream
     starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
     ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
-    counter = {"i": 0}
-    plain_interpret, plain_step = interpreter.interpret, interpreter.interpret_step
+    steps_of_launch = []
+    plain = {name: getattr(interpreter, name) for name in ("interpret", "interpret_step", "interpret_steps")}
 
-    def timed(launch):
+    def timed(launch, count):
         def wrapper(*a, **kw):
-            i = counter["i"]
+            i = len(steps_of_launch)
             starts[i].record()
             launch(*a, **kw)
             ends[i].record()
-            counter["i"] = i + 1
+            steps_of_launch.append(count(*a, **kw))
         return wrapper
 
-    interpreter.interpret, interpreter.interpret_step = timed(plain_interpret), timed(plain_step)
+    interpreter.interpret = timed(plain["interpret"], lambda *a, **kw: 1)
+    interpreter.interpret_step = timed(plain["interpret_step"], lambda *a, **kw: 1)
+    interpreter.interpret_steps = timed(plain["interpret_steps"], lambda globs, embed, token_in, tokens_out: tokens_out.numel())
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     gen.generate(output_tokens, prompt_len=prefill, ntok=args.steps, ntok_already_generated=1 + args.warmup)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    interpreter.interpret, interpreter.interpret_step = plain_interpret, plain_step
+    for name, fn in plain.items():
+        setattr(interpreter, name, fn)
     mk_mod.check_status(device)
+    assert sum(steps_of_launch) == args.steps
 
-    kernel_ms = [s.elapsed_time(e) for s, e in zip(starts, ends)]
-    kernel_ms_mean = sum(kernel_ms) / len(kernel_ms)
+    launch_ms = [s.elapsed_time(e) for s, e, _ in zip(starts, ends, steps_of_launch)]
     first_pos = prefill + args.warmup
-    bytes_per_step = sum(algorithmic_bytes(cfg, first_pos + i) for i in range(args.steps)) / args.steps
-    achieved_gbps = bytes_per_step / (kernel_ms_mean * 1e-3) / 1e9
+    step_bytes = [algorithmic_bytes(cfg, first_pos + i) for i in range(args.steps)]
+    bytes_per_step = sum(step_bytes) / args.steps
+    # the roofline is quoted on the launches of the usual size (a shorter last launch, when the
+    # step count does not divide, is left out of the mean)
+    usual = max(steps_of_launch)
+    usual_ms, usual_bytes, at = [], [], 0
+    for ms, n in zip(launch_ms, steps_of_launch):
+        if n == usual:
+            usual_ms.append(ms)
+            usual_bytes.append(sum(step_bytes[at : at + n]))
+        at += n
+    kernel_ms_mean = sum(usual_ms) / len(usual_ms)
+    bytes_per_launch = sum(usual_bytes) / len(usual_bytes)
+    achieved_gbps = bytes_per_launch / (kernel_ms_mean * 1e-3) / 1e9
 
     tokens_gpu = output_tokens[0].cpu().tolist()
 
@@ -213,7 +235,9 @@ def main():
     traffic_file = ROOT / "profiles" / f"mk_llama_kernel_{args.workload}_traffic.json"
     if traffic_file.exists():
         measured = json.loads(traffic_file.read_text())
-        traffic = measured["fetch_bytes_per_launch"] + measured["write_bytes_per_launch"]
+        # the counters were taken per launch of `steps_per_launch` steps
+        per_step = (measured["fetch_bytes_per_launch"] + measured["write_bytes_per_launch"]) / measured.get("steps_per_launch", 1)
+        traffic = int(per_step * usual)
 
     result = {
         "metric": "batch-1 decode tokens/s (Llama-3.2-1B arch)",
@@ -236,6 +260,7 @@ def main():
             "attention_partitions": partitions,
             "assignment": args.sched,
             "loop": args.loop,
+            "steps_per_launch": usual,
             "instructions_per_step": len(schedule.dag_nodes),
         },
         "roofline": {
@@ -247,7 +272,9 @@ def main():
             "traffic": traffic,
             "kernel": "mk_llama_kernel<4,4,64>",
             "kernel_us": round(kernel_ms_mean * 1e3, 2),
-            "algorithmic_bytes_per_launch": int(bytes_per_step),
+            "kernel_us_per_step": round(kernel_ms_mean * 1e3 / usual, 2),
+            "launches_timed": len(usual_ms),
+            "algorithmic_bytes_per_launch": int(bytes_per_launch),
         },
         "cpu_baseline": cpu_baseline,
         "parity": parity,

@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define MK_LLAMA_ABI_VERSION 2
+#define MK_LLAMA_ABI_VERSION 3
 #define MK_INSTRUCTION_WORDS 32   /* megakernels/scheduler.py:13, include/config.cuh:14 */
 #define MK_TIMING_SLOTS 128       /* megakernels/scheduler.py:14, include/config.cuh:18 */
 #define MK_BARRIER_ROWS 10        /* megakernels/demos/latency/scheduler.py:53-61 */
@@ -100,6 +100,13 @@ typedef struct mk_llama_args {
     const uint16_t *embed_table;          /* [vocab, hidden]; needed with token_in */
     const int64_t *token_in;              /* device; hidden_states starts as embed_table[*token_in] */
     int64_t *token_out;                   /* device; receives argmax(logits), first index on ties */
+    /* Optional: several decode steps in one launch (no counterpart in the reference, which launches
+     * once per token).  num_steps > 1 needs embed_table, token_in, token_out and
+     * MK_FLAG_RESET_BARRIERS; step s runs at position pos_id + s, starts from the token of step s - 1
+     * (*token_in for s = 0) and writes its token to token_out[s], so token_out holds num_steps
+     * entries.  0 and 1 both mean one step. */
+    int32_t num_steps;
+    int32_t reserved0;                    /* keep zero */
 } mk_llama_args;
 
 /* Bytes of scratch device memory a launch needs for these shapes.  The caller

@@ -68,7 +68,8 @@ constexpr int kQueueSlots = 256;    // longest instruction queue per worker (kep
 constexpr int kMaxHeadDim = 128;
 constexpr int kGqa = 4;             // query heads per KV head handled by one attention instruction
 constexpr int kStatusInts = 16;
-constexpr int kDoneSlot = 8;        // workspace int: workgroups finished
+constexpr int kDoneSlot = 8;        // workspace int: workgroups finished, summed over the steps of a launch
+constexpr int kStepSlot = 9;        // workspace int: decode steps of this launch completed and published
 
 // Weight rows in flight per consumer wave, per instruction kind (16 VGPRs per 2048-element row; the
 // 9-wave workgroup leaves each lane 168 VGPRs).  The rows requested before the dependency wait are
@@ -176,6 +177,9 @@ __device__ __forceinline__ uint64_t ld_u64(const void *p) {
 __device__ __forceinline__ float ld_f32(const float *p) { return mkm::bits_f32(ld_u32(p)); }
 __device__ __forceinline__ void st_u32(void *p, uint32_t v) {
     __hip_atomic_store(as_global((uint32_t *)p), v, __ATOMIC_RELAXED, AG);
+}
+__device__ __forceinline__ void st_u64(void *p, uint64_t v) {
+    __hip_atomic_store(as_global((uint64_t *)p), v, __ATOMIC_RELAXED, AG);
 }
 __device__ __forceinline__ void st_f32(float *p, float v) { st_u32(p, mkm::f32_bits(v)); }
 __device__ __forceinline__ void st_i32(int *p, int v) { __hip_atomic_store(as_global(p), v, __ATOMIC_RELAXED, AG); }
@@ -1755,124 +1759,173 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
         if (tid == kConsumerThreads) record_status(make_ctx(sm, 0, 0), MK_STATUS_BAD_TOKEN);
         refusal = MK_STATUS_BAD_TOKEN;
     }
-    for (int slot = 0; slot < a.num_slots && refusal == 0; slot++) {
-        const int opcode = sm->queue[slot][0];
-        if (opcode == 0) continue;  // NoOp pads the queues (megakernels/scheduler.py:287-289)
-        {
-            const Ctx c = make_ctx(sm, slot, opcode);
-            trace_event(c, kEvStart);
-            if (c.trace && c.controller && c.lane == 0) st_plain_i32(c.trace + kEvOpcode, opcode);
-        }
-        bool ok = true;
-        switch (opcode) {
-        case 1: ok = op_matvec<1, KC_HID>(sm, slot, &refusal); break;
-        case 2: ok = op_attention<D>(sm, slot, &refusal); break;
-        case 3: ok = op_attention_reduction<D>(sm, slot, &refusal); break;
-        case 4:
-            if constexpr (KC_HID == KC_RED && MK_PAIR_OPROJ_UPGATE) {
-                if (slot + 1 < a.num_slots && sm->queue[slot + 1][0] == 5) {
-                    const int executed = op_oproj_upgate<KC_HID>(sm, slot, &refusal);
-                    ok = executed > 0;
-                    slot += ok ? executed - 1 : 0;
-                    break;
-                }
-            }
-            ok = op_matvec<4, KC_RED>(sm, slot, &refusal);
-            break;
-        case 5: ok = op_matvec<5, KC_HID>(sm, slot, &refusal); break;
-        case 6: ok = op_matvec<6, KC_RED>(sm, slot, &refusal); break;
-        case 7: ok = op_lm_head<KC_HID>(sm, slot, &refusal); break;
-        default: ok = bail(make_ctx(sm, slot, opcode), MK_STATUS_BAD_OPCODE, &refusal);  // reference: trap, include/util.cuh:38
-        }
-        if (!ok) break;
-        trace_event(make_ctx(sm, slot, sm->queue[slot][0]), kEvEnd);
-    }
-    if (refusal && tid == 0) sm->abort = refusal;
-
-    // The last workgroup to get here folds the sharded counters into `barriers` and leaves the
-    // shards zeroed for the next launch.
-    wait_stores();
-    wg_barrier();
+    // A launch covers one decode step, or `num_steps` of them back to back: the token a step
+    // produces starts the next one, at the next position.
+    const int steps = a.num_steps > 1 ? a.num_steps : 1;
     const WsLayout wl = ws_layout(a.num_layers, a.hidden_size, a.intermediate_size, a.matvec_reduction_size);
     int *status = static_cast<int *>(a.workspace) + wl.status;
-    if (tid == 0) {
-        const int done = __hip_atomic_fetch_add(&status[kDoneSlot], 1, __ATOMIC_RELAXED, AG);
-        sm->last_flag = done == (int)gridDim.x - 1;
-    }
-    wg_barrier();
-    if (sm->last_flag) {
-        // One thread per (counter, shard), two pairs per trip with both loads in flight, and the
-        // workers' maxima requested before the fold: the step's token waits for one round trip here,
-        // not for a chain of them.
-        const int counters = a.num_layers * kHotRows;
-        int *shards = static_cast<int *>(a.workspace) + wl.shards;
-        const int cols = a.num_attention_heads + 2 * a.num_kv_heads;
-        const bool reset = (a.flags & MK_FLAG_RESET_BARRIERS) != 0;
-        int *maxima = static_cast<int *>(a.workspace) + wl.argmax;
-        constexpr int kMaxTrips = (kMaxWorkers + kThreads - 1) / kThreads;
-        uint64_t reported[kMaxTrips];
-#pragma unroll
-        for (int k = 0; k < kMaxTrips; k++) {
-            const int w = tid + k * kThreads;
-            reported[k] = a.token_out && w < (int)gridDim.x ? ld_u64(maxima + 2 * w) : 0;
+    for (int step = 0; step < steps; step++) {
+        for (int slot = 0; slot < a.num_slots && refusal == 0; slot++) {
+            const int opcode = sm->queue[slot][0];
+            if (opcode == 0) continue;  // NoOp pads the queues (megakernels/scheduler.py:287-289)
+            {
+                const Ctx c = make_ctx(sm, slot, opcode);
+                trace_event(c, kEvStart);
+                if (c.trace && c.controller && c.lane == 0) st_plain_i32(c.trace + kEvOpcode, opcode);
+            }
+            bool ok = true;
+            switch (opcode) {
+            case 1: ok = op_matvec<1, KC_HID>(sm, slot, &refusal); break;
+            case 2: ok = op_attention<D>(sm, slot, &refusal); break;
+            case 3: ok = op_attention_reduction<D>(sm, slot, &refusal); break;
+            case 4:
+                if constexpr (KC_HID == KC_RED && MK_PAIR_OPROJ_UPGATE) {
+                    if (slot + 1 < a.num_slots && sm->queue[slot + 1][0] == 5) {
+                        const int executed = op_oproj_upgate<KC_HID>(sm, slot, &refusal);
+                        ok = executed > 0;
+                        slot += ok ? executed - 1 : 0;
+                        break;
+                    }
+                }
+                ok = op_matvec<4, KC_RED>(sm, slot, &refusal);
+                break;
+            case 5: ok = op_matvec<5, KC_HID>(sm, slot, &refusal); break;
+            case 6: ok = op_matvec<6, KC_RED>(sm, slot, &refusal); break;
+            case 7: ok = op_lm_head<KC_HID>(sm, slot, &refusal); break;
+            default: ok = bail(make_ctx(sm, slot, opcode), MK_STATUS_BAD_OPCODE, &refusal);  // reference: trap, include/util.cuh:38
+            }
+            if (!ok) break;
+            trace_event(make_ctx(sm, slot, sm->queue[slot][0]), kEvEnd);
         }
-        auto shard_at = [&](int k) {
-            const int i = k / kShards, sh = k % kShards;
-            return kShardPad ? shards + ((size_t)i * kShards + sh) * kShardPad : shards + (size_t)sh * counters + i;
-        };
-        auto fold = [&](int k, int v) {
-            if (v == 0) return;
-            st_i32(shard_at(k), 0);
-            const int i = k / kShards;
-            if (!reset) add_i32(a.barriers + ((size_t)(i / kHotRows) * MK_BARRIER_ROWS + 2 + i % kHotRows) * cols, v);
-        };
-        const int pairs = counters * kShards;
-        for (int k = tid; k < pairs; k += 2 * kThreads) {
-            const int k2 = k + kThreads;
-            const int v = ld_i32(shard_at(k));
-            const int v2 = k2 < pairs ? ld_i32(shard_at(k2)) : 0;
-            fold(k, v);
-            if (k2 < pairs) fold(k2, v2);
+        if (refusal && tid == 0) sm->abort = refusal;
+
+        // End of a step.  The last workgroup to get here folds the sharded counters into `barriers`
+        // (or zeroes `barriers`), leaves the shards zeroed, and turns the workers' LM-head maxima into
+        // the step's token.  With more steps to go it then publishes the step, and everybody else
+        // waits for that before starting on the next token.
+        wait_stores();
+        wg_barrier();
+        if (tid == 0) {
+            const int done = __hip_atomic_fetch_add(&status[kDoneSlot], 1, __ATOMIC_RELAXED, AG);
+            sm->last_flag = done == (int)gridDim.x * (step + 1) - 1;
         }
-        if (reset) {
-            const int words = a.num_layers * MK_BARRIER_ROWS * cols;
-            for (int i = tid; i < words; i += kThreads) st_i32(a.barriers + i, 0);
-        }
-        if (a.token_out) {
-            // the workers' LM-head maxima -> the step's token
-            float v = -INFINITY;
-            int idx = INT_MAX;
+        wg_barrier();
+        const bool more = step + 1 < steps && sm->abort == 0;
+        if (sm->last_flag) {
+            // One thread per (counter, shard), two pairs per trip with both loads in flight, and the
+            // workers' maxima requested before the fold: the step's token waits for one round trip
+            // here, not for a chain of them.
+            const int counters = a.num_layers * kHotRows;
+            int *shards = static_cast<int *>(a.workspace) + wl.shards;
+            const int cols = a.num_attention_heads + 2 * a.num_kv_heads;
+            const bool reset = (a.flags & MK_FLAG_RESET_BARRIERS) != 0;
+            int *maxima = static_cast<int *>(a.workspace) + wl.argmax;
+            constexpr int kMaxTrips = (kMaxWorkers + kThreads - 1) / kThreads;
+            uint64_t reported[kMaxTrips];
 #pragma unroll
             for (int k = 0; k < kMaxTrips; k++) {
-                const int stored = (int)(reported[k] >> 32);
-                if (stored) {
-                    const float wv = __builtin_bit_cast(float, (int)(uint32_t)reported[k]);
-                    if (wv > v || (wv == v && stored - 1 < idx)) {
-                        v = wv;
-                        idx = stored - 1;
+                const int w = tid + k * kThreads;
+                reported[k] = a.token_out && w < (int)gridDim.x ? ld_u64(maxima + 2 * w) : 0;
+            }
+            auto shard_at = [&](int k) {
+                const int i = k / kShards, sh = k % kShards;
+                return kShardPad ? shards + ((size_t)i * kShards + sh) * kShardPad : shards + (size_t)sh * counters + i;
+            };
+            auto fold = [&](int k, int v) {
+                if (v == 0) return;
+                st_i32(shard_at(k), 0);
+                const int i = k / kShards;
+                if (!reset) add_i32(a.barriers + ((size_t)(i / kHotRows) * MK_BARRIER_ROWS + 2 + i % kHotRows) * cols, v);
+            };
+            const int pairs = counters * kShards;
+            for (int k = tid; k < pairs; k += 2 * kThreads) {
+                const int k2 = k + kThreads;
+                const int v = ld_i32(shard_at(k));
+                const int v2 = k2 < pairs ? ld_i32(shard_at(k2)) : 0;
+                fold(k, v);
+                if (k2 < pairs) fold(k2, v2);
+            }
+            if (reset) {
+                const int words = a.num_layers * MK_BARRIER_ROWS * cols;
+                for (int i = tid; i < words; i += kThreads) st_i32(a.barriers + i, 0);
+            }
+            if (a.token_out) {
+                // the workers' LM-head maxima -> the step's token
+                float v = -INFINITY;
+                int idx = INT_MAX;
+#pragma unroll
+                for (int k = 0; k < kMaxTrips; k++) {
+                    const int stored = (int)(reported[k] >> 32);
+                    if (stored) {
+                        const float wv = __builtin_bit_cast(float, (int)(uint32_t)reported[k]);
+                        if (wv > v || (wv == v && stored - 1 < idx)) {
+                            v = wv;
+                            idx = stored - 1;
+                        }
+                        st_i32(maxima + 2 * (tid + k * kThreads) + 1, 0);
                     }
-                    st_i32(maxima + 2 * (tid + k * kThreads) + 1, 0);
+                }
+                argmax_combine_wave(v, idx);
+                if (tid % 64 == 0) {
+                    sm->out[2 * (tid / 64)] = v;
+                    sm->flags[tid / 64] = idx;
+                }
+                wg_barrier();
+                if (tid == 0) {
+                    for (int w = 1; w < kThreads / 64; w++) {
+                        const float wv = sm->out[2 * w];
+                        const int wi = sm->flags[w];
+                        if (wv > v || (wv == v && wi < idx)) {
+                            v = wv;
+                            idx = wi;
+                        }
+                    }
+                    const int token = idx == INT_MAX ? 0 : idx;
+                    st_u64(a.token_out + step, (uint64_t)token);
+                    sm->token = token;
                 }
             }
-            argmax_combine_wave(v, idx);
-            if (tid % 64 == 0) {
-                sm->out[2 * (tid / 64)] = v;
-                sm->flags[tid / 64] = idx;
+            if (more) {
+                // everything the next step relies on (zeroed counters, the token) has landed before
+                // the step is published
+                wait_stores();
+                wg_barrier();
+                if (tid == 0) st_i32(&status[kStepSlot], step + 1);
+            } else if (tid == 0) {
+                st_i32(&status[kDoneSlot], 0);
+                st_i32(&status[kStepSlot], 0);
             }
-            wg_barrier();
+        } else if (more && tid < 64) {
+            // one wave watches for the step's publication (and for a failure anywhere)
+            const long long t0 = wall_clock64();
+            const long long limit = (long long)(a.spin_limit_us ? a.spin_limit_us : 2000000u) * 100;
+            bool ok = true;
+            while (true) {
+                const int published = ld_i32(&status[kStepSlot]);
+                const int failure = ld_i32(&status[0]);
+                if (failure != 0) {
+                    ok = false;
+                    break;
+                }
+                if (published > step) break;
+                if (wall_clock64() - t0 > limit) {
+                    if (tid == 0) record_status(make_ctx(sm, 0, 0), MK_STATUS_BARRIER_TIMEOUT);
+                    ok = false;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(MK_POLL_SLEEP);
+            }
+            compiler_fence();
+            const uint64_t token = ok ? ld_u64(a.token_out + step) : 0;
             if (tid == 0) {
-                for (int w = 1; w < kThreads / 64; w++) {
-                    const float wv = sm->out[2 * w];
-                    const int wi = sm->flags[w];
-                    if (wv > v || (wv == v && wi < idx)) {
-                        v = wv;
-                        idx = wi;
-                    }
-                }
-                *as_global(a.token_out) = idx == INT_MAX ? 0 : (long long)idx;
+                if (ok) sm->token = (int)token;
+                else sm->abort = 1;
             }
         }
-        if (tid == 0) st_i32(&status[kDoneSlot], 0);
+        if (!more) break;
+        if (tid == 0) sm->args.pos_id = a.pos_id + step + 1;
+        wg_barrier();
+        if (sm->abort) break;
     }
 }
 
@@ -1973,6 +2026,15 @@ int mk_llama_launch(const mk_llama_args *args, void *hip_stream) {
             return fail(-2, "embed_table must be 16-byte aligned and token_in 8-byte aligned");
     }
     if (a.token_out && (uintptr_t)a.token_out % 8) return fail(-2, "token_out must be 8-byte aligned");
+    if (a.num_steps < 0) return fail(-3, "num_steps must not be negative");
+    if (a.num_steps > 1) {
+        if (!a.token_in || !a.token_out || !(a.flags & MK_FLAG_RESET_BARRIERS))
+            return fail(-3, "several steps per launch need token_in, token_out and MK_FLAG_RESET_BARRIERS");
+        const long long last = (long long)a.pos_id + a.num_steps - 1;
+        if (last >= a.kv_max_len || last >= a.rope_positions)
+            return fail(-4, "%d steps from position %d run past the KV cache (%d) or rope table (%d)", a.num_steps,
+                        a.pos_id, a.kv_max_len, a.rope_positions);
+    }
     // weight rows are addressed as 32-bit offsets into one buffer per matrix
     const uint64_t widest = 2ull * hid * (uint64_t)(a.vocab_size > a.intermediate_size ? a.vocab_size : a.intermediate_size);
     if (widest >= (1ull << 31)) return fail(-3, "a weight matrix of %llu bytes exceeds the 2 GiB a buffer can address", (unsigned long long)widest);

@@ -46,6 +46,7 @@ class MkLlamaArgs(ctypes.Structure):
         + [("workspace", _P), ("workspace_bytes", ctypes.c_uint64),
            ("spin_limit_us", ctypes.c_uint32), ("flags", ctypes.c_uint32)]
         + [("embed_table", _P), ("token_in", _P), ("token_out", _P)]
+        + [("num_steps", _I), ("reserved0", _I)]
     )
 
 
@@ -99,9 +100,10 @@ def _check(t: torch.Tensor, dtype: torch.dtype, name: str) -> int:
     return t.data_ptr()
 
 
-def _token_pointer(t, name):
-    if not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype != torch.int64 or t.numel() != 1:
-        raise RuntimeError(f"{name} must be a one-element int64 device tensor")
+def _token_pointer(t, name, count=1):
+    if (not isinstance(t, torch.Tensor) or not t.is_cuda or t.dtype != torch.int64 or t.numel() != count
+            or not t.is_contiguous()):
+        raise RuntimeError(f"{name} must be a contiguous int64 device tensor of {count} element(s)")
     return t.data_ptr()
 
 
@@ -115,7 +117,7 @@ def mk_llama(
     pos_id, attn_scale, rms_norm_eps, skip_attn_reduction,
     stream=None,
     *,
-    embed_table=None, token_in=None, token_out=None, reset_barriers=False,
+    embed_table=None, token_in=None, token_out=None, reset_barriers=False, num_steps=1,
 ):
     """Launch one decode step asynchronously on ``stream`` (a torch stream;
     default: the current one).  Shapes are taken from the tensors.
@@ -125,7 +127,10 @@ def mk_llama(
     are one-element int64 device tensors (views into the token buffer) - the
     step starts from ``embed_table[token_in]`` instead of ``hidden_states`` and
     writes ``argmax(logits)`` to ``token_out``; ``reset_barriers`` leaves
-    ``barriers`` zeroed for the next launch."""
+    ``barriers`` zeroed for the next launch.  ``num_steps`` > 1 runs that many
+    decode steps in the one launch: step ``s`` works at position ``pos_id + s``
+    from the token of step ``s - 1`` and writes ``token_out[s]`` (``token_out``
+    then has ``num_steps`` elements)."""
     lib = load_library()
     bf, f32, i32 = torch.bfloat16, torch.float32, torch.int32
     a = MkLlamaArgs()
@@ -207,8 +212,12 @@ def mk_llama(
             raise RuntimeError("token_in needs embed_table of shape [vocab, hidden]")
         a.embed_table = _check(embed_table, bf, "embed_table")
         a.token_in = _token_pointer(token_in, "token_in")
+    num_steps = int(num_steps)
+    if num_steps < 1:
+        raise RuntimeError("num_steps must be at least 1")
     if token_out is not None:
-        a.token_out = _token_pointer(token_out, "token_out")
+        a.token_out = _token_pointer(token_out, "token_out", num_steps)
+    a.num_steps = num_steps
 
     if stream is None:
         stream = torch.cuda.current_stream(barriers.device)

@@ -70,3 +70,11 @@ class LatencyMK_Interpreter(MK_Interpreter):
         the launch, ``megakernels/generators.py:121-143``)."""
         interpret_with_mk(globs, self.mk_func, embed_table=embed_table, token_in=token_in,
                           token_out=token_out, reset_barriers=True)
+
+    def interpret_steps(self, globs: Globals, embed_table, token_in, tokens_out):
+        """``len(tokens_out)`` decode steps in one launch, starting at
+        ``globs.pos_id``: step ``s`` consumes the token of step ``s - 1``
+        (``token_in`` for the first) and writes ``tokens_out[s]``.  The
+        reference launches once per token (``megakernels/generators.py:121-143``)."""
+        interpret_with_mk(globs, self.mk_func, embed_table=embed_table, token_in=token_in,
+                          token_out=tokens_out, reset_barriers=True, num_steps=tokens_out.numel())

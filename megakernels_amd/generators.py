@@ -73,6 +73,7 @@ class MK_Generator(Generator):
         skip_mk: bool = False,
         skip_rest: bool = False,
         fused_step: bool | None = None,
+        steps_per_launch: int = 0,
     ):
         self.model = model
         self.interpreter = interpreter
@@ -85,6 +86,9 @@ class MK_Generator(Generator):
         # kernels around the launch.
         can_fuse = hasattr(interpreter, "interpret_step") and barrier_fill_val == 0 and not skip_mk and not skip_rest
         self.fused_step = can_fuse if fused_step is None else (fused_step and can_fuse)
+        # With the glue folded in, consecutive steps need nothing from the host: `generate` hands the
+        # interpreter up to this many steps per launch (0: all of them, 1: one launch per token).
+        self.steps_per_launch = steps_per_launch if hasattr(interpreter, "interpret_steps") else 1
         self.fill()
 
     def fill(self):
@@ -111,10 +115,17 @@ class MK_Generator(Generator):
             globs = self.schedule.globs
             embed = self.model.model.embed_tokens.weight
             self.fill()
-            for i in range(ntok):
+            i = 0
+            while i < ntok:
+                n = ntok - i if self.steps_per_launch <= 0 else min(self.steps_per_launch, ntok - i)
                 src = ntok_already_generated + i - 1
                 globs.pos_id = prompt_len + ntok_already_generated + i - 1
-                self.interpreter.interpret_step(globs, embed, output_tokens[0, src : src + 1], output_tokens[0, src + 1 : src + 2])
+                if n == 1:
+                    self.interpreter.interpret_step(globs, embed, output_tokens[0, src : src + 1], output_tokens[0, src + 1 : src + 2])
+                else:
+                    self.interpreter.interpret_steps(globs, embed, output_tokens[0, src : src + 1], output_tokens[0, src + 1 : src + 1 + n])
+                    globs.pos_id += n - 1  # the position the launch ended on
+                i += n
             return
         for i in range(ntok):
             src = ntok_already_generated + i - 1

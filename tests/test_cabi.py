@@ -51,7 +51,7 @@ def test_workspace_size_and_static_queries():
     assert small == 4 * (32 + 16 * 16 * 4 + 128 + 128 + 2 * 1024 + 4 * 2048)
     assert big > small and big < (1 << 20)
     assert lib.mk_llama_workspace_bytes(0, 2048, 8192, 2048) == 0
-    assert lib.mk_llama_query(3) == 2                      # ABI version
+    assert lib.mk_llama_query(3) == 3                      # ABI version
     assert lib.mk_llama_query(2) == 576                    # 8 consumer waves + 1 controller wave
     assert 80 * 1024 < lib.mk_llama_query(1) <= 160 * 1024  # one workgroup per CU, within gfx950's LDS
     assert lib.mk_llama_query(4) >= 2048
@@ -88,7 +88,7 @@ def test_python_args_struct_matches_the_header():
             names.append(re.findall(r"(\w+)\s*$", part.strip())[0])
     assert names == [f[0] for f in mk_llama.MkLlamaArgs._fields_]
     # 23 pointers, pos_id + 2 floats + flag, 14 int shapes, workspace ptr + u64 + 2 x u32, 3 optional pointers
-    assert ctypes.sizeof(mk_llama.MkLlamaArgs) == 23 * 8 + 4 * 4 + 14 * 4 + 8 + 8 + 8 + 3 * 8
+    assert ctypes.sizeof(mk_llama.MkLlamaArgs) == 23 * 8 + 4 * 4 + 14 * 4 + 8 + 8 + 8 + 3 * 8 + 2 * 4
 
 
 SHIM = r"""

@@ -21,7 +21,7 @@ def _interpreter():
     return LatencyMK_Interpreter(), sys.modules["mk_llama"]
 
 
-def _decode_case(cfg, workers, prefill, ntok, partitions=1, max_len=256, sched="rr", fused=False):
+def _decode_case(cfg, workers, prefill, ntok, partitions=1, max_len=256, sched="rr", fused=False, steps_per_launch=1):
     from megakernels_amd.generators import MK_Generator
     from oracle import pyvm
 
@@ -39,8 +39,8 @@ def _decode_case(cfg, workers, prefill, ntok, partitions=1, max_len=256, sched="
 
     tokens_gpu = torch.zeros(1, ntok + 1, dtype=torch.long, device="cuda:0")
     tokens_gpu[0, 0] = 5
-    gen = MK_Generator(model_gpu, interp, schedule_gpu, fused_step=fused)
-    assert gen.fused_step == fused
+    gen = MK_Generator(model_gpu, interp, schedule_gpu, fused_step=fused, steps_per_launch=steps_per_launch)
+    assert gen.fused_step == fused and gen.steps_per_launch == steps_per_launch
     gen.generate(tokens_gpu, prompt_len=prefill, ntok=ntok)
     mk_mod.check_status("cuda:0")
     assert tokens_gpu.cpu().tolist() == tokens_cpu.tolist()
@@ -75,6 +75,44 @@ def test_decode_1b_slice_many_steps_split_kv_one_launch_per_token():
     # 160 consecutive launches, every one checked through its token: a race between workgroups would
     # have many chances to show
     _decode_case(config_1b_slice(layers=2), workers=256, prefill=500, ntok=160, partitions=3, max_len=1024, fused=True)
+
+
+def test_decode_tiny_all_steps_in_one_launch():
+    _decode_case(config_tiny(), workers=16, prefill=20, ntok=12, fused=True, steps_per_launch=0)
+
+
+def test_decode_tiny_split_kv_seven_steps_per_launch():
+    # launches of 7, 7 and 6 steps; positions 30..49 cross the 16-token block boundaries at 32 and 48
+    _decode_case(config_tiny(), workers=16, prefill=30, ntok=20, partitions=3, fused=True, steps_per_launch=7)
+
+
+def test_decode_1b_slice_all_steps_in_one_launch():
+    _decode_case(config_1b_slice(layers=3), workers=256, prefill=100, ntok=8, fused=True, steps_per_launch=0)
+
+
+def test_decode_1b_slice_many_steps_split_kv_in_one_launch():
+    # 160 steps without leaving the kernel: every step's token is checked, and every step starts
+    # behind a grid-wide hand-over of the previous token
+    _decode_case(config_1b_slice(layers=2), workers=256, prefill=500, ntok=160, partitions=3, max_len=1024, fused=True,
+                 steps_per_launch=0)
+
+
+def test_decode_8b_slice_all_steps_in_one_launch():
+    _decode_case(config_8b_slice(layers=2), workers=256, prefill=50, ntok=4, partitions=2, fused=True, steps_per_launch=0)
+
+
+def test_steps_past_the_kv_cache_are_refused():
+    from megakernels_amd.generators import MK_Generator
+
+    cfg = config_tiny()
+    model = make_model(cfg, max_len=32)
+    fill_kv(model, upto=8)
+    schedule = build_schedule(model, 16)
+    model_gpu, schedule_gpu = mirror_to_gpu(model, schedule)
+    interp, _ = _interpreter()
+    tokens = torch.zeros(1, 64, dtype=torch.long, device="cuda:0")
+    with pytest.raises(RuntimeError, match="run past the KV cache"):
+        MK_Generator(model_gpu, interp, schedule_gpu, fused_step=True).generate(tokens, prompt_len=8, ntok=40)
 
 
 def test_token_outside_the_vocabulary_is_reported():
