@@ -214,8 +214,8 @@ def test_unsatisfiable_dependency_times_out_and_reports():
 
 
 def test_missing_attention_partials_time_out_in_the_merge():
-    """Split-KV schedule without its attention instructions: the merging waves poll tagged values that
-    never arrive, give up at the spin limit and the whole grid drains."""
+    """Split-KV schedule without its attention instructions: the merge waits for partition counters
+    that never move, gives up at the spin limit and the whole grid drains."""
     model = make_model(config_tiny())
     fill_kv(model, upto=40)
     schedule = build_schedule(model, 16, partitions=2)
@@ -232,6 +232,32 @@ def test_missing_attention_partials_time_out_in_the_merge():
         mk_mod.spin_limit_us = 0
     assert code == 1 and opcode in (3, 4)
     test_decode_tiny_split_kv_crossing_block_boundaries()
+
+
+def test_failure_in_a_launch_of_several_steps_drains_the_grid():
+    """The same broken schedule inside a launch of four steps: the workers that give up never reach the
+    end of the step, the others find the failure while waiting for the step to be published, and no
+    second step starts."""
+    from megakernels_amd.generators import MK_Generator
+
+    model = make_model(config_tiny())
+    fill_kv(model, upto=40)
+    schedule = build_schedule(model, 16, partitions=2)
+    g = schedule.globs
+    g.instructions[g.instructions[:, :, 0] == 2] = 0
+    model_gpu, schedule_gpu = mirror_to_gpu(model, schedule)
+    interp, mk_mod = _interpreter()
+    tokens = torch.full((1, 5), -1, dtype=torch.long, device="cuda:0")
+    tokens[0, 0] = 5
+    mk_mod.spin_limit_us = 20000
+    try:
+        MK_Generator(model_gpu, interp, schedule_gpu, fused_step=True, steps_per_launch=0).generate(tokens, prompt_len=40, ntok=4)
+        code, worker, slot, opcode = mk_mod.read_status("cuda:0")
+    finally:
+        mk_mod.spin_limit_us = 0
+    assert code == 1 and opcode in (3, 4)
+    assert tokens[0, 2:].tolist() == [-1, -1, -1]      # nothing after the first step was produced
+    test_decode_tiny_all_steps_in_one_launch()
 
 
 def test_unknown_opcode_and_bad_fields_are_reported():
