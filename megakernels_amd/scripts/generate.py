@@ -4,9 +4,10 @@
     python -m megakernels_amd.scripts.generate mode=mk ntok=100
     python -m megakernels_amd.scripts.generate .l8 mode=mk prompt_len=32 ntok=64 num_attention_partitions=4
 
-Differences forced by the environment: there is no tokenizer or checkpoint download, so the prompt is
-``prompt_len`` seeded random token ids and ``model`` is ``1b`` / ``8b`` (random-initialised architecture)
-or a local checkpoint directory.  Modes: ``mk`` (HIP megakernel) and ``torch`` (plain PyTorch forward).
+Differences forced by the environment: nothing is downloaded, so ``model`` is ``1b`` / ``8b``
+(random-initialised architecture; the prompt is ``prompt_len`` seeded random token ids) or a local checkpoint
+directory; when that directory holds a tokenizer, ``prompt=...`` (``chat=true`` for the chat template) is
+tokenised and the output is printed as text too, as the reference does (``generate.py:98-112,186-202``).  Modes: ``mk`` (HIP megakernel) and ``torch`` (plain PyTorch forward).
 As in the reference (``generate.py:125-137``) the prompt is prefilled by the PyTorch model and the timed
 region is ``ntok - 1`` decode steps, repeated ``num_warmup + num_iters`` times.
 """
@@ -26,12 +27,16 @@ from megakernels_amd.llama import LlamaConfig, LlamaForCausalLM
 from megakernels_amd.mk import DEFAULT_MK_DIR
 from megakernels_amd.model_types import BatchState, ExtraModelConfig
 from megakernels_amd.scheduler import assign_to_sms, tensorize_instructions
+from megakernels_amd.scripts.text import encode_prompt, load_tokenizer
 
 
 @dataclass
 class ScriptConfig:
     model: str = "1b"
     device: str = "cuda:0"
+    prompt: str = "tell me a funny joke about cookies"
+    chat: bool = False
+    token_details: bool = False
     prompt_len: int = 32
     ntok: int = 100
     mode: str = "mk"
@@ -108,9 +113,13 @@ def load_model(config: ScriptConfig) -> LlamaForCausalLM:
 def main(config: ScriptConfig):
     torch.cuda.set_device(config.device)
     model = load_model(config)
-    gen_ids = torch.Generator().manual_seed(config.seed + 1)
-    input_ids = torch.randint(0, model.config.vocab_size, (1, config.prompt_len), generator=gen_ids).to(model.device)
-    prompt_len = config.prompt_len
+    tokenizer = None if config.model in ("1b", "8b") else load_tokenizer(config.model)
+    if tokenizer is not None:
+        input_ids = encode_prompt(tokenizer, config.prompt, config.chat).to(model.device)
+    else:
+        gen_ids = torch.Generator().manual_seed(config.seed + 1)
+        input_ids = torch.randint(0, model.config.vocab_size, (1, config.prompt_len), generator=gen_ids).to(model.device)
+    prompt_len = input_ids.shape[-1]
     print(f"Input ids shape: {tuple(input_ids.shape)}")
 
     prefill = model(BatchState(input_ids=input_ids, position_ids=torch.arange(prompt_len, device=model.device)))
@@ -152,6 +161,12 @@ def main(config: ScriptConfig):
     print(f"Average time: {elapsed * 1000:.2f}ms (CPU: {elapsed_cpu * 1000:.2f}ms)")
     if config.tokens:
         print("Output ids: ", output_tokens.cpu())
+        if tokenizer is not None:
+            print("Output text: ", tokenizer.batch_decode(output_tokens.cpu()))
+    if config.token_details and tokenizer is not None:
+        print("More detailed output (output id, position id, token):")
+        for i, token in enumerate(tokenizer.convert_ids_to_tokens(output_tokens[0].cpu().tolist())):
+            print(f"  {i:5d} {i + prompt_len:6d}  {token}")
     fwd_per_second = (config.ntok - 1) / elapsed
     print(f"Fwd per second: {fwd_per_second:.2f}")
     print(f"Tokens per second: {fwd_per_second:.2f}")

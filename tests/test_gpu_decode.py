@@ -21,13 +21,15 @@ def _interpreter():
     return LatencyMK_Interpreter(), sys.modules["mk_llama"]
 
 
-def _decode_case(cfg, workers, prefill, ntok, partitions=1, max_len=256, sched="rr", fused=False, steps_per_launch=1):
+def _decode_case(cfg, workers, prefill, ntok, partitions=1, max_len=256, sched="rr", fused=False, steps_per_launch=1,
+                 model=None):
     from megakernels_amd.generators import MK_Generator
     from oracle import pyvm
 
     print(f"decode case hidden={cfg.hidden_size} workers={workers} prefill={prefill} ntok={ntok} "
           f"partitions={partitions}", flush=True)
-    model = make_model(cfg, max_len=max_len)
+    if model is None:
+        model = make_model(cfg, max_len=max_len)
     fill_kv(model, upto=prefill)
     schedule = build_schedule(model, workers, partitions=partitions, sched=sched)
     model_gpu, schedule_gpu = mirror_to_gpu(model, schedule)
@@ -99,6 +101,26 @@ def test_decode_1b_slice_many_steps_split_kv_in_one_launch():
 
 def test_decode_8b_slice_all_steps_in_one_launch():
     _decode_case(config_8b_slice(layers=2), workers=256, prefill=50, ntok=4, partitions=2, fused=True, steps_per_launch=0)
+
+
+def test_decode_from_a_hugging_face_checkpoint(tmp_path):
+    """The whole user path: a checkpoint directory written by the installed third-party `transformers`
+    (untied head, llama3 rope scaling), loaded with `from_pretrained`, decoded through the megakernel,
+    token-exact against the checker."""
+    transformers = pytest.importorskip("transformers")
+    from megakernels_amd.llama import LlamaForCausalLM
+    from megakernels_amd.model_types import ExtraModelConfig
+
+    hf_cfg = transformers.LlamaConfig(
+        vocab_size=1024, hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=8,
+        num_key_value_heads=2, head_dim=64, max_position_embeddings=256, rms_norm_eps=1e-5, rope_theta=500000.0,
+        tie_word_embeddings=False, attention_bias=False, mlp_bias=False,
+        rope_scaling={"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                      "original_max_position_embeddings": 64})
+    torch.manual_seed(17)
+    transformers.LlamaForCausalLM(hf_cfg).eval().save_pretrained(tmp_path, safe_serialization=True)
+    model = LlamaForCausalLM.from_pretrained(tmp_path, ExtraModelConfig(interleave_rope=True, max_len_override=128))
+    _decode_case(model.config, workers=16, prefill=24, ntok=10, partitions=2, fused=True, steps_per_launch=0, model=model)
 
 
 def test_steps_past_the_kv_cache_are_refused():

@@ -250,3 +250,74 @@ def test_from_pretrained_reads_a_hugging_face_checkpoint_and_matches_its_forward
 def _final_norm(model, hidden):
     w = model.lm_head.input_norm.weight.float()
     return w * hidden * torch.rsqrt(hidden.pow(2).mean(-1, keepdim=True) + model.config.rms_norm_eps)
+
+
+def _tiny_chat_checkpoint(tmp_path):
+    """A checkpoint directory as a user would have it: weights and config written by the installed
+    third-party `transformers`, a word-level tokenizer with a chat template, a generation config."""
+    transformers = pytest.importorskip("transformers")
+    tokenizers = pytest.importorskip("tokenizers")
+    words = ["<pad>", "<bos>", "<eos>", "<user>", "<assistant>", "hi", "tell", "me", "a", "joke", "about", "cookies",
+             "why", "did", "the", "cookie", "cry"]
+    vocab = {w: i for i, w in enumerate(words)}
+    tok = tokenizers.Tokenizer(tokenizers.models.WordLevel(vocab, unk_token="<pad>"))
+    tok.pre_tokenizer = tokenizers.pre_tokenizers.WhitespaceSplit()
+    fast = transformers.PreTrainedTokenizerFast(tokenizer_object=tok, bos_token="<bos>", eos_token="<eos>", pad_token="<pad>")
+    fast.chat_template = ("<bos>{% for m in messages %} <{{ m['role'] }}> {{ m['content'] }} <eos>{% endfor %}"
+                          "{% if add_generation_prompt %} <assistant>{% endif %}")
+    fast.save_pretrained(tmp_path)
+    hf_cfg = transformers.LlamaConfig(
+        vocab_size=64, hidden_size=128, intermediate_size=256, num_hidden_layers=2, num_attention_heads=2,
+        num_key_value_heads=1, head_dim=64, max_position_embeddings=128, rms_norm_eps=1e-5, rope_theta=500000.0,
+        tie_word_embeddings=True, attention_bias=False, mlp_bias=False, eos_token_id=2, bos_token_id=1)
+    torch.manual_seed(3)
+    transformers.LlamaForCausalLM(hf_cfg).eval().save_pretrained(tmp_path, safe_serialization=True)
+    (tmp_path / "generation_config.json").write_text('{"eos_token_id": [2, 0]}')
+    return vocab
+
+
+def test_prompt_encoding_and_eos_ids_of_a_local_checkpoint(tmp_path):
+    from megakernels_amd.scripts.text import encode_messages, encode_prompt, eos_token_ids, load_tokenizer
+
+    vocab = _tiny_chat_checkpoint(tmp_path)
+    assert load_tokenizer(tmp_path / "nowhere") is None
+    tok = load_tokenizer(tmp_path)
+    plain = encode_prompt(tok, "tell me a joke", chat=False)
+    assert plain.tolist() == [[vocab[w] for w in "tell me a joke".split()]]
+    chat = encode_prompt(tok, "tell me a joke", chat=True)
+    want = "<bos> <user> tell me a joke <eos> <assistant>".split()
+    assert chat.tolist() == [[vocab[w] for w in want]]
+    two = encode_messages(tok, [{"role": "user", "content": "hi"}, {"role": "assistant", "content": "why"},
+                                {"role": "user", "content": "joke"}])
+    assert two.shape[1] == 1 + 3 * 2 + 3 + 1
+    assert eos_token_ids(tmp_path, tok) == [2, 0]
+    (tmp_path / "generation_config.json").unlink()
+    assert eos_token_ids(tmp_path, tok) == [2]          # from config.json
+
+
+def test_repl_conversation_on_the_pytorch_generator(tmp_path):
+    """The chat loop's core with the plain PyTorch generator on the CPU: each turn re-renders the whole
+    conversation, stops at an end-of-sequence id, and a second turn sees the first one's answer."""
+    from megakernels_amd.generators import PyTorchGenerator
+    from megakernels_amd.scripts.llama_repl import Conversation, parse_args
+    from megakernels_amd.scripts.text import eos_token_ids, load_tokenizer
+
+    _tiny_chat_checkpoint(tmp_path)
+    tok = load_tokenizer(tmp_path)
+    model = LlamaForCausalLM.from_pretrained(tmp_path, ExtraModelConfig(interleave_rope=True, max_len_override=96))
+    chat = Conversation(model, PyTorchGenerator(model), tok, eos_token_ids(tmp_path, tok), max_tokens_per_turn=24)
+    text, generated, seconds = chat.say("tell me a joke about cookies")
+    assert isinstance(text, str) and 1 <= generated <= 23 and seconds > 0
+    ids = chat.output_tokens[0].tolist()
+    stops = [i for i, t in enumerate(ids[: generated + 1]) if t in (0, 2)]
+    # the reply ends at the first end-of-sequence id, if one was produced within the chunks that ran
+    assert text == tok.decode(ids[: stops[0] if stops else 24], skip_special_tokens=True)
+    first_len = len(chat.messages)
+    chat.say("why")
+    assert first_len == 2 and len(chat.messages) == 4 and chat.messages[1]["role"] == "assistant"
+    with pytest.raises(RuntimeError, match="does not fit the KV cache"):
+        Conversation(model, PyTorchGenerator(model), tok, [2], max_tokens_per_turn=200).say("hi")
+    cfg = parse_args([f"model={tmp_path}", "mode=torch", "max_tokens_per_turn=8", "print_prompt_len=true"])
+    assert cfg.mode == "torch" and cfg.max_tokens_per_turn == 8 and cfg.print_prompt_len is True
+    with pytest.raises(SystemExit):
+        parse_args(["mode=mk"])
