@@ -29,6 +29,10 @@
 //     `barriers`, so after the launch the tensor holds exactly the reference VM's counts.
 //   * every barrier wait is bounded (spin_limit_us): on expiry the worker records a status
 //     code and every workgroup leaves its instruction loop, so the grid always drains.
+//   * optionally the per-token glue of the reference's decode loop is part of the launch (embedding
+//     row of the input token, argmax of the logits, barrier reset), and then a launch can run
+//     several decode steps back to back: the last workgroup of a step publishes the step's token,
+//     the others wait for that and start over one position further on.
 //
 // Arithmetic: bit-compatible with a fixed "column order" so results can be compared exactly
 // with a CPU restatement of the Python VM.  A dot product over K elements is computed by one
