@@ -59,11 +59,11 @@ constexpr int kThreads = kConsumerThreads + 64;  // + one controller wave
 #ifndef MK_SHARDS
 #define MK_SHARDS 16
 #endif
-#ifndef MK_SHARD_PAD
-#define MK_SHARD_PAD 0
-#endif
 constexpr int kShards = MK_SHARDS;   // shards per hot barrier counter
-constexpr int kShardPad = MK_SHARD_PAD;  // 0: shard-major planes; n > 0: counter-major, n ints per shard
+#ifndef MK_REPLICAS
+#define MK_REPLICAS 4
+#endif
+constexpr int kReplicas = MK_REPLICAS;  // copies of every shard: a signal goes to all, a worker polls one
 constexpr int kHotRows = 4;         // barrier rows 2..5 are sharded
 constexpr int kOutRows = 2048;      // rows staged in LDS between matvec and epilogue
 constexpr int kMaxK = 4096;         // longest activation vector handed through LDS
@@ -121,7 +121,7 @@ __host__ __device__ inline WsLayout ws_layout(int L, int hid, int inter, int R) 
     size_t off = 0;
     w.status = off;   off += kStatusInts;
     off = (off + 31) & ~(size_t)31;  // counters start on a 128-byte line
-    w.shards = off;   off += (size_t)kShards * L * kHotRows * (kShardPad ? kShardPad : 1);
+    w.shards = off;   off += (size_t)kReplicas * kShards * L * kHotRows;
     w.arrive_o = off; off += hid / 16;
     w.arrive_d = off; off += hid / 16;
     w.argmax = off;   off += 2 * (size_t)kMaxWorkers;  // per worker: value bits, index + 1 (0: nothing)
@@ -436,9 +436,10 @@ __device__ __forceinline__ int *bar_ptr(const Ctx &c, int layer, int row, int co
     const int cols = uni(a.num_attention_heads) + 2 * uni(a.num_kv_heads);
     return uni(a.barriers) + ((size_t)layer * MK_BARRIER_ROWS + row) * cols + col;
 }
-__device__ __forceinline__ int *shard_ptr(const Ctx &c, int shard, int layer, int row) {
-    if (kShardPad) return ws_shards(c) + ((size_t)(layer * kHotRows + (row - 2)) * kShards + shard) * kShardPad;
-    return ws_shards(c) + ((size_t)shard * uni(c.sm->args.num_layers) + layer) * kHotRows + (row - 2);
+// [replica][shard][layer][row]: the shards of one counter lie in different cache lines
+__device__ __forceinline__ int *shard_ptr(const Ctx &c, int replica, int shard, int layer, int row) {
+    const int L = uni(c.sm->args.num_layers);
+    return ws_shards(c) + (((size_t)replica * kShards + shard) * L + layer) * kHotRows + (row - 2);
 }
 
 // first error wins
@@ -502,7 +503,9 @@ __device__ bool poll_counters(const Ctx &c, const int *ptr, bool sum_mode, int t
 }
 
 __device__ __forceinline__ const int *sharded_lane_ptr(const Ctx &c, int layer, int row) {
-    if (c.lane < kShards) return shard_ptr(c, c.lane, layer, row);
+    // 256 workers reading the same 16 lines every quarter microsecond queue up at those lines'
+    // memory channels; with four copies each line has a quarter of the readers
+    if (c.lane < kShards) return shard_ptr(c, (c.worker / kShards) % kReplicas, c.lane, layer, row);
     if (c.lane == kShards) return bar_ptr(c, layer, row, 0);
     return nullptr;
 }
@@ -512,7 +515,8 @@ __device__ __forceinline__ bool poll_sharded(const Ctx &c, int layer, int row, i
 
 // one arrival on a sharded counter; the caller has waited for its stores
 __device__ __forceinline__ void signal_sharded_lane(const Ctx &c, int layer, int row, int count) {
-    add_i32(shard_ptr(c, c.worker & (kShards - 1), layer, row), count);
+#pragma unroll
+    for (int r = 0; r < kReplicas; r++) add_i32(shard_ptr(c, r, c.worker & (kShards - 1), layer, row), count);
 }
 __device__ __forceinline__ void signal_sharded(const Ctx &c, int layer, int row, int count) {
     if (c.lane == 0) signal_sharded_lane(c, layer, row, count);
@@ -1831,17 +1835,15 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
                 const int w = tid + k * kThreads;
                 reported[k] = a.token_out && w < (int)gridDim.x ? ld_u64(maxima + 2 * w) : 0;
             }
-            auto shard_at = [&](int k) {
-                const int i = k / kShards, sh = k % kShards;
-                return kShardPad ? shards + ((size_t)i * kShards + sh) * kShardPad : shards + (size_t)sh * counters + i;
-            };
+            // k = (replica, shard, counter); every copy is zeroed, the first one is what gets counted
+            auto shard_at = [&](int k) { return shards + k; };
             auto fold = [&](int k, int v) {
                 if (v == 0) return;
                 st_i32(shard_at(k), 0);
-                const int i = k / kShards;
-                if (!reset) add_i32(a.barriers + ((size_t)(i / kHotRows) * MK_BARRIER_ROWS + 2 + i % kHotRows) * cols, v);
+                const int i = k % counters;
+                if (!reset && k < counters * kShards) add_i32(a.barriers + ((size_t)(i / kHotRows) * MK_BARRIER_ROWS + 2 + i % kHotRows) * cols, v);
             };
-            const int pairs = counters * kShards;
+            const int pairs = counters * kShards * kReplicas;
             for (int k = tid; k < pairs; k += 2 * kThreads) {
                 const int k2 = k + kThreads;
                 const int v = ld_i32(shard_at(k));
