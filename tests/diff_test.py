@@ -5,6 +5,10 @@ difference, the mean relative difference and the number of differing elements.  
 
     python tests/diff_test.py model=1b layer_limit=1 stop_after_op=oproj prompt_len=10 ntok=10
     python tests/diff_test.py model=tiny .full num_attention_partitions=3
+    python tests/diff_test.py model=1b layer_limit=1 start_after_op=oproj
+
+``start_after_op`` (reference ``diff_test.py:122-152,198-208``): the checker runs the instructions up to and
+including that op on both sets of buffers, the megakernel gets only the rest.
 
 It lives with the tests because it drives the checker, which the product never imports.
 """
@@ -30,6 +34,7 @@ class ScriptConfig:
     prompt_len: int = 10
     ntok: int = 10
     stop_after_op: str | None = None
+    start_after_op: str | None = None
     layer_limit: int | None = 1
     sched: str = "rr"
     workers: int = 256
@@ -80,13 +85,25 @@ def main(config: ScriptConfig):
     g.hidden_states.normal_()
     g.pos_id = seq_len - 1
     g.barriers.fill_(config.barrier_init_val)
+    instructions = schedule.get_linear_instructions()
+    if config.start_after_op is not None:
+        from megakernels_amd.scheduler import assign_to_sms, tensorize_instructions
+
+        head = build_schedule(model, config.workers, partitions=config.num_attention_partitions, sched=config.sched,
+                              stop_after_op=config.start_after_op, layer_limit=config.layer_limit).get_linear_instructions()
+        assert len(head) < len(instructions) and instructions[: len(head)] == head, "start_after_op must come before the end"
+        print(f"running the first {len(head)} of {len(instructions)} instructions with the checker...")
+        pyvm.interpret(g, head, check_barriers=config.barrier_init_val == 0)
+        instructions = instructions[len(head):]
+        tensorize_instructions(g, assign_to_sms("rr", instructions=instructions, sm_count=config.workers))
     if config.noops:
         g.instructions.zero_()
     queue_lengths = [int((q[:, 0] != 0).sum()) for q in g.instructions]
     print(f"worker queue lengths: min={min(queue_lengths)}, max={max(queue_lengths)}, "
           f"mean={sum(queue_lengths) / len(queue_lengths):.2f}")
     _, schedule_gpu = mirror_to_gpu(model, schedule)
-    instructions = [] if config.noops else schedule.get_linear_instructions()
+    if config.noops:
+        instructions = []
     pyvm.interpret(g, instructions, check_barriers=config.barrier_init_val == 0)
     interp = LatencyMK_Interpreter()
     interp.interpret(schedule_gpu.globs)

@@ -86,3 +86,46 @@ def test_8b_slice_column_groups():
 
 def test_8b_slice_split_kv():
     _one_step_case(config_8b_slice(), workers=256, pos=1500, partitions=8, max_len=2048)
+
+
+def _suffix_case(cfg, workers, pos, start_after_op, partitions=1):
+    """The reference's diff_test `start_after_op` (scripts/diff_test.py:122-152,198-208): the first part
+    of a layer is run by the checker on both sets of buffers, the megakernel then gets only the
+    instructions after it - its waits are satisfied by counts that were already in `barriers` when
+    it started, its inputs were written by somebody else."""
+    from megakernels_amd.scheduler import assign_to_sms, tensorize_instructions
+    from oracle import pyvm
+
+    print(f"suffix case hidden={cfg.hidden_size} workers={workers} pos={pos} start_after_op={start_after_op} "
+          f"partitions={partitions}", flush=True)
+    model = make_model(cfg)
+    fill_kv(model, upto=pos)
+    whole = build_schedule(model, workers, partitions=partitions, layer_limit=1)
+    first = build_schedule(model, workers, partitions=partitions, layer_limit=1, stop_after_op=start_after_op)
+    everything, head = whole.get_linear_instructions(), first.get_linear_instructions()
+    assert 0 < len(head) < len(everything) and everything[: len(head)] == head
+    tail = everything[len(head):]
+    g = whole.globs
+    g.hidden_states.copy_(torch.randn(cfg.hidden_size, generator=torch.Generator().manual_seed(13)).to(torch.bfloat16))
+    g.pos_id = pos
+    pyvm.interpret(g, head)
+    tensorize_instructions(g, assign_to_sms("rr", instructions=tail, sm_count=workers))
+    model_gpu, schedule_gpu = mirror_to_gpu(model, whole)
+    assert int(schedule_gpu.globs.barriers.sum()) > 0
+    pyvm.interpret(g, tail)
+    _gpu_step(schedule_gpu)
+    report = mismatches(g, schedule_gpu.globs)
+    assert not report, f"tensors differ from the checker: {report}"
+
+
+@pytest.mark.parametrize("start_after_op", ["qkv", "partial", "oproj", "upgate"])
+def test_tiny_layer_started_after_an_op(start_after_op):
+    _suffix_case(config_tiny(), workers=16, pos=21, start_after_op=start_after_op)
+
+
+def test_tiny_split_kv_layer_started_after_the_reduction():
+    _suffix_case(config_tiny(), workers=16, pos=44, start_after_op="reduction", partitions=3)
+
+
+def test_1b_slice_layer_started_after_the_o_projection():
+    _suffix_case(config_1b_slice(layers=2), workers=256, pos=70, start_after_op="oproj")
