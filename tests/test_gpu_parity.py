@@ -129,3 +129,38 @@ def test_tiny_split_kv_layer_started_after_the_reduction():
 
 def test_1b_slice_layer_started_after_the_o_projection():
     _suffix_case(config_1b_slice(layers=2), workers=256, pos=70, start_after_op="oproj")
+
+
+def _tiny_long_context():
+    cfg = config_tiny()
+    cfg.max_position_embeddings = 8192      # length of the rotary tables
+    return cfg
+
+
+def test_tiny_partition_of_exactly_the_on_chip_limit():
+    """One partition over 4096 cached positions fills the score buffer to the last slot."""
+    _one_step_case(_tiny_long_context(), workers=16, pos=4095, max_len=4096 + 8)
+
+
+def test_partition_beyond_the_on_chip_limit_is_reported():
+    import sys
+
+    cfg = _tiny_long_context()
+    model = make_model(cfg, max_len=4096 + 64)
+    fill_kv(model, upto=4100)
+    schedule = build_schedule(model, 16)
+    schedule.globs.pos_id = 4100                       # 4101 positions in one partition
+    _, schedule_gpu = mirror_to_gpu(model, schedule)
+    from megakernels_amd.demos.latency.mk import LatencyMK_Interpreter
+
+    mk_mod_interp = LatencyMK_Interpreter()
+    mk_mod = sys.modules["mk_llama"]
+    mk_mod.spin_limit_us = 20000
+    try:
+        mk_mod_interp.interpret(schedule_gpu.globs)
+        code, worker, slot, opcode = mk_mod.read_status("cuda:0")
+    finally:
+        mk_mod.spin_limit_us = 0
+    assert code == 3 and opcode == 2
+    # and the same context split in two partitions is fine
+    _one_step_case(cfg, workers=16, pos=4100, partitions=2, max_len=4096 + 64)
