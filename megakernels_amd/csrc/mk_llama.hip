@@ -112,9 +112,13 @@ constexpr int rows_in_flight(int wanted) { return KC <= 4 ? wanted : (wanted < 2
 // workspace layout (ints unless noted)
 // ---------------------------------------------------------------------------------------------
 struct WsLayout {
-    size_t status, shards, arrive_o, arrive_d, argmax, partial, total_bytes;
+    size_t status, shards, arrive_o, arrive_d, argmax, partial, pads, total_bytes;
 };
 constexpr int kMaxWorkers = 1024;   // workers that can report an LM-head maximum
+constexpr int kPadInts = 32;        // a padded counter owns a 128-byte line
+// upper bound of the barrier tensor's columns (query + key + value heads) for a hidden size: heads
+// are at least 64 wide and four query heads share a KV head
+__host__ __device__ constexpr int pad_cols(int hid) { return hid / 64 + hid / 128; }
 
 __host__ __device__ inline WsLayout ws_layout(int L, int hid, int inter, int R) {
     WsLayout w;
@@ -129,6 +133,9 @@ __host__ __device__ inline WsLayout ws_layout(int L, int hid, int inter, int R) 
     w.partial = off;  // floats: [max(groups_o, groups_d)][hid]
     int g_o = hid / R, g_d = inter / R;
     off += (size_t)(g_o > g_d ? g_o : g_d) * hid;
+    // the per-head counters (barrier rows 0 and 1), one cache line each
+    off = (off + 31) & ~(size_t)31;
+    w.pads = off;     off += (size_t)L * 2 * pad_cols(hid) * kPadInts;
     w.total_bytes = off * 4;
     return w;
 }
@@ -437,6 +444,14 @@ __device__ __forceinline__ int *bar_ptr(const Ctx &c, int layer, int row, int co
     return uni(a.barriers) + ((size_t)layer * MK_BARRIER_ROWS + row) * cols + col;
 }
 // [replica][shard][layer][row]: the shards of one counter lie in different cache lines
+// Barrier rows 0 (QKV blocks per head) and 1 (attention partitions per head) while the kernel runs.
+// In `barriers` the counters of all heads share two cache lines; hundreds of arrivals within a
+// microsecond then queue up behind each other (same-line atomics are served one at a time) and
+// the waiting side sees its own head complete late.  Here every counter has a line of its own.
+__device__ __forceinline__ int *pad_ptr(const Ctx &c, int layer, int row, int col) {
+    ArgsRef a = c.sm->args;
+    return ws_ints(c) + ws_regions(c).pads + ((size_t)(layer * 2 + row) * pad_cols(uni(a.hidden_size)) + col) * kPadInts;
+}
 __device__ __forceinline__ int *shard_ptr(const Ctx &c, int replica, int shard, int layer, int row) {
     const int L = uni(c.sm->args.num_layers);
     return ws_shards(c) + (((size_t)replica * kShards + shard) * L + layer) * kHotRows + (row - 2);
@@ -457,11 +472,13 @@ __device__ void record_status(const Ctx &c, int code) {
 struct PollTicket {
     const int *ptr;
     int value, status;
+    int base;  // what the counter's word in `barriers` held when the launch started (it does not move during one)
 };
-__device__ __forceinline__ PollTicket poll_issue(const Ctx &c, const int *ptr) {
+__device__ __forceinline__ PollTicket poll_issue(const Ctx &c, const int *ptr, const int *in_barriers = nullptr) {
     PollTicket t;
     t.ptr = ptr;
     t.value = ptr ? ld_i32(ptr) : 0;
+    t.base = in_barriers ? ld_i32(in_barriers) : 0;
     t.status = c.lane == 63 ? ld_i32(ws_status(c)) : 0;
     return t;
 }
@@ -480,7 +497,7 @@ __device__ __forceinline__ bool poll_wait(const Ctx &c, PollTicket t, bool sum_m
     int v = t.value, st = t.status;
     bool first = true;
     while (true) {
-        const bool ok = sum_mode ? (lane_sum_i32(v) >= target) : (bool)__all(t.ptr == nullptr || v >= target);
+        const bool ok = sum_mode ? (lane_sum_i32(v) >= target) : (bool)__all(t.ptr == nullptr || v + t.base >= target);
         if (ok) break;
         if (first) not_yet();
         first = false;
@@ -498,8 +515,8 @@ __device__ __forceinline__ bool poll_wait(const Ctx &c, PollTicket t, bool sum_m
     compiler_fence();  // data loads stay after the successful poll
     return true;
 }
-__device__ bool poll_counters(const Ctx &c, const int *ptr, bool sum_mode, int target) {
-    return poll_wait(c, poll_issue(c, ptr), sum_mode, target, []() {});
+__device__ bool poll_counters(const Ctx &c, const int *ptr, const int *in_barriers, bool sum_mode, int target) {
+    return poll_wait(c, poll_issue(c, ptr, in_barriers), sum_mode, target, []() {});
 }
 
 __device__ __forceinline__ const int *sharded_lane_ptr(const Ctx &c, int layer, int row) {
@@ -510,7 +527,7 @@ __device__ __forceinline__ const int *sharded_lane_ptr(const Ctx &c, int layer, 
     return nullptr;
 }
 __device__ __forceinline__ bool poll_sharded(const Ctx &c, int layer, int row, int target) {
-    return poll_counters(c, sharded_lane_ptr(c, layer, row), true, target);
+    return poll_counters(c, sharded_lane_ptr(c, layer, row), nullptr, true, target);
 }
 
 // one arrival on a sharded counter; the caller has waited for its stores
@@ -953,7 +970,7 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
             }
             wait_stores();
             // one arrival per block on its head's counter (python_vm.py:248)
-            for (int b = c.lane; b < nblk; b += 64) add_i32(bar_ptr(c, layer, 0, (start + b) / (D / 16)), 1);
+            for (int b = c.lane; b < nblk; b += 64) add_i32(pad_ptr(c, layer, 0, (start + b) / (D / 16)), 1);
         });
 }
 
@@ -1388,11 +1405,10 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
 
     if (c.controller) {
         // wait: Q heads, K head and V head of this step are complete (python_vm.py:281-290)
-        const int *p = nullptr;
-        if (c.lane < G) p = bar_ptr(c, layer, 0, h0 + c.lane);
-        else if (c.lane == G) p = bar_ptr(c, layer, 0, H + kvh);
-        else if (c.lane == G + 1) p = bar_ptr(c, layer, 0, H + KVH + kvh);
-        const bool ok = poll_counters(c, p, false, D / 16);
+        const int col = c.lane < G ? h0 + c.lane : c.lane == G ? H + kvh : H + KVH + kvh;
+        const bool mine = c.lane < G + 2;
+        const bool ok = poll_counters(c, mine ? pad_ptr(c, layer, 0, col) : nullptr, mine ? bar_ptr(c, layer, 0, col) : nullptr,
+                                      false, D / 16);
         trace_event(c, kEvDepReady);
         if (!barrier_inputs_ready(c, ok)) return false;
         wg_barrier();  // wave maxima
@@ -1626,7 +1642,7 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
         trace_consumer(c, 31);
         if (d == 0) {
             if (skip) signal_sharded_lane(c, layer, 2, 1);
-            else add_i32(bar_ptr(c, layer, 1, head), 1);
+            else add_i32(pad_ptr(c, layer, 1, head), 1);
         }
         trace_consumer_flush(c, 29, 31);
     }
@@ -1657,8 +1673,9 @@ static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot
     if (bad) return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
 
     if (c.controller) {
-        const int *p = c.lane < R ? bar_ptr(c, layer, 1, hs + c.lane) : nullptr;
-        const bool ok = poll_counters(c, p, false, P);
+        const bool mine = c.lane < R;
+        const bool ok = poll_counters(c, mine ? pad_ptr(c, layer, 1, hs + c.lane) : nullptr,
+                                      mine ? bar_ptr(c, layer, 1, hs + c.lane) : nullptr, false, P);
         trace_event(c, kEvDepReady);
         if (!barrier_inputs_ready(c, ok)) return false;
         trace_event(c, kEvComputeDone);
@@ -1851,6 +1868,28 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
                 fold(k, v);
                 if (k2 < pairs) fold(k2, v2);
             }
+            {
+                // the padded per-head counters, four looks in flight per thread and trip
+                int *pads = static_cast<int *>(a.workspace) + wl.pads;
+                const int pc = pad_cols(a.hidden_size), npad = a.num_layers * 2 * pc;
+                for (int k0 = tid; k0 < npad; k0 += 4 * kThreads) {
+                    int v[4];
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        const int k = k0 + u * kThreads;
+                        v[u] = k < npad ? ld_i32(pads + (size_t)k * kPadInts) : 0;
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; u++) {
+                        const int k = k0 + u * kThreads;
+                        if (v[u] == 0) continue;
+                        st_i32(pads + (size_t)k * kPadInts, 0);
+                        const int col = k % pc, lr = k / pc;
+                        if (!reset && col < cols)
+                            add_i32(a.barriers + ((size_t)(lr / 2) * MK_BARRIER_ROWS + lr % 2) * cols + col, v[u]);
+                    }
+                }
+            }
             if (reset) {
                 const int words = a.num_layers * MK_BARRIER_ROWS * cols;
                 for (int i = tid; i < words; i += kThreads) st_i32(a.barriers + i, 0);
@@ -2018,6 +2057,7 @@ int mk_llama_launch(const mk_llama_args *args, void *hip_stream) {
         return fail(-3, "unsupported head grouping: %d query heads for %d KV heads (need %d per KV head)",
                     a.num_attention_heads, a.num_kv_heads, kGqa);
     if (a.num_attention_heads * D != hid) return fail(-3, "num_attention_heads * head_dim must equal hidden_size");
+    if (D < 64) return fail(-3, "head_dim must be at least 64");
     if (a.attn_reduction_size != kGqa) return fail(-3, "attn_reduction_size must be %d", kGqa);
     if (R <= 0 || hid % R || a.intermediate_size % R) return fail(-3, "sizes are not multiples of the reduction width");
     if (a.vocab_size % 16 || a.intermediate_size % 16) return fail(-3, "vocab and intermediate sizes must be multiples of 16");

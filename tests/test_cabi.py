@@ -48,7 +48,7 @@ def test_workspace_size_and_static_queries():
     big = lib.mk_llama_workspace_bytes(32, 4096, 14336, 2048)
     # 1B: status padded to a 128-byte line + 16 shards x 16 layers x 4 counters + 2 x 128 arrival counters
     # + 1024 x 2 LM-head maxima + 4 x 2048 partial sums
-    assert small == 4 * (32 + 4 * 16 * 16 * 4 + 128 + 128 + 2 * 1024 + 4 * 2048)
+    assert small == 4 * (32 + 4 * 16 * 16 * 4 + 128 + 128 + 2 * 1024 + 4 * 2048 + 16 * 2 * 48 * 32)
     assert big > small and big < (1 << 20)
     assert lib.mk_llama_workspace_bytes(0, 2048, 8192, 2048) == 0
     assert lib.mk_llama_query(3) == 3                      # ABI version
