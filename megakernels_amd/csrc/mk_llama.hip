@@ -1051,11 +1051,25 @@ __device__ __forceinline__ bool control_matvec_add(const Ctx &c) {
                     const int row0 = start * 16 + p * 2;
                     const uint32_t h = prefetched ? (p < 64 ? pre[0] : pre[1]) : ld_u32(resid + row0);
                     float lo = mkm::bf16_lo(h), hi = mkm::bf16_hi(h);
-                    for (int g = 0; g < ngroups; g++) {
-                        const uint64_t v = ld_u64(partial + (size_t)g * hid + row0);
+                    auto apply = [&](uint64_t v) {
                         lo = mkm::round_bf16(lo + mkm::bits_f32((uint32_t)v));
                         hi = mkm::round_bf16(hi + mkm::bits_f32((uint32_t)(v >> 32)));
+                    };
+                    // The partials are applied in group order, but requested four (then two) at a time:
+                    // this worker is the one the next layer is waiting for, and a loop over the
+                    // groups would pay one round trip per group.
+                    const float *mine = partial + row0;
+                    int g = 0;
+                    for (; g + 4 <= ngroups; g += 4) {
+                        const uint64_t v0 = ld_u64(mine + (size_t)g * hid), v1 = ld_u64(mine + (size_t)(g + 1) * hid);
+                        const uint64_t v2 = ld_u64(mine + (size_t)(g + 2) * hid), v3 = ld_u64(mine + (size_t)(g + 3) * hid);
+                        apply(v0); apply(v1); apply(v2); apply(v3);
                     }
+                    for (; g + 2 <= ngroups; g += 2) {
+                        const uint64_t v0 = ld_u64(mine + (size_t)g * hid), v1 = ld_u64(mine + (size_t)(g + 1) * hid);
+                        apply(v0); apply(v1);
+                    }
+                    if (g < ngroups) apply(ld_u64(mine + (size_t)g * hid));
                     st_u32(resid + row0, mkm::pack_bf16(lo, hi));
                 }
             }
