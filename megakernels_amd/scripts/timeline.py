@@ -1,15 +1,17 @@
 """Per-instruction timeline of one decode step, from the megakernel's own timing records.
 
-    python -m megakernels_amd.scripts.timeline [layers=16] [pos=4100] [partitions=0] [layer=1] [out=trace.npz]
+    python -m megakernels_amd.scripts.timeline [model=1b] [layers=16] [pos=4100] [partitions=0] [layer=1]
+                                               [sched=rr] [out=trace.npz]
 
-Builds the random-initialised 1B architecture with ``layers`` layers, fills the KV cache up to ``pos``
+Builds the random-initialised 1B (or ``model=8b``) architecture with ``layers`` layers, fills the KV cache up to ``pos``
 with seeded noise, runs a few warm-up steps, then one step with ``MK_FLAG_TIMINGS`` set and prints,
 per instruction kind, how long the workers waited for the dependency, loaded the activation vector,
 computed and wrote back; and for one layer when each kind started, saw its dependency and ended across
 the workers.  ``out=`` saves the raw records (``timings`` [workers, slots, 128] and ``instructions``
 [workers, slots, 32], plain ``numpy`` arrays) for a Gantt view elsewhere - the counterpart of the
-reference's ``diff_test.py outfile=`` dump (``scripts/diff_test.py:231-242``).  The reference records the same events (``include/util.cuh:215-246``) when compiled with
-``TIMING_RECORD_ENABLED``; here the records are taken on request at run time.
+reference's ``diff_test.py outfile=`` dump (``scripts/diff_test.py:231-242``).  The reference records the
+same events (``include/util.cuh:215-246``) when compiled with ``TIMING_RECORD_ENABLED``; here the records
+are taken on request at run time.
 
 Times are microseconds since the workgroup started (100 MHz wall clock of the device).
 """
@@ -32,16 +34,18 @@ NAMES = {1: "qkv", 2: "attention", 3: "merge", 4: "o-proj", 5: "up/gate", 6: "do
 
 
 def main(argv):
-    opts = {"layers": 16, "pos": 4100, "partitions": 0, "layer": 1, "sched": "rr", "out": ""}
+    opts = {"model": "1b", "layers": 16, "pos": 4100, "partitions": 0, "layer": 1, "sched": "rr", "out": ""}
     for arg in argv:
         key, _, value = arg.partition("=")
         if key not in opts:
             raise SystemExit(f"unknown option {key}; known: {', '.join(opts)}")
-        opts[key] = value if key in ("sched", "out") else int(value)
+        opts[key] = value if key in ("model", "sched", "out") else int(value)
     if not torch.cuda.is_available():
         raise SystemExit("timeline needs a GPU")
     device = torch.device("cuda:0")
-    cfg = LlamaConfig.llama_1b()
+    if opts["model"] not in ("1b", "8b"):
+        raise SystemExit("model is 1b or 8b")
+    cfg = LlamaConfig.llama_1b() if opts["model"] == "1b" else LlamaConfig.llama_8b()
     cfg.num_hidden_layers = opts["layers"]
     pos = opts["pos"]
     model = LlamaForCausalLM.from_random(cfg, ExtraModelConfig(interleave_rope=True, max_len_override=pos + 64), seed=0)
@@ -83,7 +87,7 @@ def main(argv):
     if opts["out"]:
         np.savez_compressed(opts["out"], timings=globs.timings.cpu().numpy(), instructions=ins,
                             ticks_per_microsecond=np.array(100))
-    print(f"{opts['layers']} layers, position {pos}, {partitions} attention partitions, {workers} workers, "
+    print(f"{opts['model']}, {opts['layers']} layers, position {pos}, {partitions} attention partitions, {workers} workers, "
           f"assignment {opts['sched']}: kernel {start.elapsed_time(end) * 1e3:.1f} us with timing records on, "
           f"last instruction ends at {t[:, :, 4].max():.1f} us")
     print("\nper instruction kind, mean / max over all instructions (us):")
