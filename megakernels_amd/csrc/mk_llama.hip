@@ -103,6 +103,9 @@ constexpr int rows_in_flight(int wanted) { return KC <= 4 ? wanted : (wanted < 2
 #ifndef MK_PAIR_OPROJ_UPGATE
 #define MK_PAIR_OPROJ_UPGATE 1      // O-proj and a directly following up/gate run as one handler
 #endif
+#ifndef MK_PARK_UPGATE
+#define MK_PARK_UPGATE 1            // long-waiting O-proj + up/gate workers park up/gate's last rows in LDS
+#endif
 #ifndef MK_POLL_SLEEP
 #define MK_POLL_SLEEP 10            // units of 64 clocks between two looks at a dependency
 #endif
@@ -1152,11 +1155,36 @@ __device__ __forceinline__ void request_rows(const Ctx &c, uint4 (&pool)[NBUF][K
         load_row<KC>(pool[Map::at(s)], matvec_row(d, c.wave + (first + s) * kConsumerWaves), present && first + s < mine, c.lane);
 }
 
+// Rows parked in LDS: the data goes from HBM straight into this wave's slice of the attention score
+// buffer (no registers involved), 16 bytes per lane and chunk, chunk j of a row at byte j * 1024.
+template <int KC, int J = 0>
+__device__ __forceinline__ void park_chunks(__amdgpu_buffer_rsrc_t rsrc, MK_LDS unsigned char *dst, uint32_t off) {
+    if constexpr (J < KC) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (MK_LDS void *)dst, 16, off, 0, J * 1024, MK_STREAM_AUX);
+        park_chunks<KC, J + 1>(rsrc, dst, off);
+    }
+}
+// request rows first, first + 1, ... first + N - 1 of this wave into its LDS slice
+template <int KC, int N>
+__device__ __forceinline__ void park_rows(const Ctx &c, MK_LDS unsigned char *slice, const MatvecDesc &d, int first, int mine,
+                                          bool present) {
+#pragma unroll
+    for (int r = 0; r < N; r++) {
+        const RowRef row = matvec_row(d, c.wave + (first + r) * kConsumerWaves);
+        const uint32_t off = present && first + r < mine ? row.offset + c.lane * 16 : kNoRow;
+        const __amdgpu_buffer_rsrc_t rsrc =
+            __builtin_amdgcn_make_buffer_rsrc((void *)uni(row.buffer.base), 0, uni((int)row.buffer.bytes), 0x00020000);
+        park_chunks<KC>(rsrc, slice + r * (KC * 1024), off);
+    }
+}
+
 // One instruction, its first Map::size rows already requested into the listed buffers: wait for the
 // activation vector, stream the rows (Map::size in flight), leave the results in LDS, and wait until
-// the controller has sent them.
-template <int KC, class Map, int NBUF>
-__device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&pool)[NBUF][KC], const MatvecDesc &d, int mine) {
+// the controller has sent them.  PARKED > 0: the instruction has at most Map::size + PARKED rows per
+// wave and those beyond the buffers were parked in `slice` on entry, so nothing is requested here.
+template <int KC, class Map, int NBUF, int PARKED = 0>
+__device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&pool)[NBUF][KC], const MatvecDesc &d, int mine,
+                                             MK_LDS const unsigned char *slice = nullptr) {
     constexpr int PF = Map::size;
     if (!barrier_inputs_ready(c, true)) return false;
     trace_consumer(c, 22);
@@ -1169,7 +1197,7 @@ __device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&pool)[NBUF][K
     };
     int base = 0;
     // rounds that are followed by more rows: every row of the round exists, every buffer is refilled
-    for (; base + PF < mine; base += PF) {
+    for (; PARKED == 0 && base + PF < mine; base += PF) {
 #pragma unroll
         for (int s = 0; s < PF; s++) {
             consume(pool[Map::at(s)], base + s);
@@ -1184,6 +1212,20 @@ __device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&pool)[NBUF][K
 #pragma unroll
     for (int s = 0; s < PF; s++)
         if (base + s < mine) consume(pool[Map::at(s)], base + s);
+    if constexpr (PARKED > 0) {
+        wait_stores();  // the parked rows were requested long ago; this makes their arrival in LDS certain
+#pragma unroll
+        for (int r = 0; r < PARKED; r++)
+            if (PF + r < mine) {
+                uint4 row[KC];
+#pragma unroll
+                for (int j = 0; j < KC; j++) {
+                    const u32x4 v = *(const MK_LDS u32x4 *)(slice + r * (KC * 1024) + j * 1024 + c.lane * 16);
+                    row[j] = uint4{v.x, v.y, v.z, v.w};
+                }
+                consume(row, PF + r);
+            }
+    }
     trace_consumer(c, 23);
     wg_barrier();  // results are in LDS
     // hold further weight requests back until the controller has sent this instruction's results and
@@ -1241,9 +1283,14 @@ static __device__ __noinline__ bool op_matvec(SmemPtr lds, int slot, int *refusa
 // are requested together with the O-proj rows, and the two O-proj buffers go to up/gate as soon as
 // O-proj is done.  Returns the number of instructions executed (2, or 1 when the second instruction
 // is malformed and left to report itself), 0 on failure.
-template <int KC>
+template <int KC, bool PARK>
 static __device__ __noinline__ int op_oproj_upgate(SmemPtr lds, int slot, int *refusal) {
     constexpr int NBUF = 6;
+    // PARK: this worker has a long wait ahead (it came here without attention work) and its up/gate
+    // instruction has at most two rows per wave beyond the six buffers: those go to LDS on entry - the
+    // attention score buffer is free - and up/gate then needs nothing from HBM once its dependency resolves
+    constexpr int kParked = PARK ? 2 : 0;
+    static_assert(!PARK || (size_t)kConsumerWaves * kParked * KC * 1024 <= sizeof(Smem::scores), "parked rows fit the score buffer");
     typedef BufMap<0, 1> MapO;
     typedef BufMap<2, 3, 4, 5> MapU0;        // requested on entry
     typedef BufMap<0, 1> MapU1;              // requested when O-proj is done
@@ -1271,11 +1318,13 @@ static __device__ __noinline__ int op_oproj_upgate(SmemPtr lds, int slot, int *r
     wg_barrier();  // entry of O-proj: the controller's first requests are out
     request_rows<KC, MapO>(co, pool, dso, 0, mine_o);
     request_rows<KC, MapU0>(co, pool, dsu, 0, mine_u, pair);
+    MK_LDS unsigned char *slice = (MK_LDS unsigned char *)&lds->scores[0][0] + co.wave * (kParked * KC * 1024);
+    if constexpr (PARK) park_rows<KC, kParked>(co, slice, dsu, MapU::size, mine_u, pair);
     if (!consumer_run<KC, MapO>(co, pool, dso, mine_o)) return 0;
     request_rows<KC, MapU1>(co, pool, dsu, MapU0::size, mine_u, pair);
     if (!pair) return 1;
     wg_barrier();  // entry of up/gate: its first requests went out long ago
-    return consumer_run<KC, MapU>(cu, pool, dsu, mine_u) ? 2 : 0;
+    return consumer_run<KC, MapU, NBUF, kParked>(cu, pool, dsu, mine_u, slice) ? 2 : 0;
 }
 
 // (value, index) pairs: the larger value wins, the smaller index on equal values - the first maximum,
@@ -1820,7 +1869,12 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
             case 4:
                 if constexpr (KC_HID == KC_RED && MK_PAIR_OPROJ_UPGATE) {
                     if (slot + 1 < a.num_slots && sm->queue[slot + 1][0] == 5) {
-                        const int executed = op_oproj_upgate<KC_HID>(sm, slot, &refusal);
+                        // rows can be parked when the wait is long (no attention just before) and the
+                        // up/gate instruction is small enough (two list entries: eight rows per wave)
+                        const bool park = MK_PARK_UPGATE && (slot == 0 || sm->queue[slot - 1][0] != 2) &&
+                                          sm->queue[slot + 1][2] >= 0 && sm->queue[slot + 1][2] <= 2;
+                        const int executed = park ? op_oproj_upgate<KC_HID, true>(sm, slot, &refusal)
+                                                  : op_oproj_upgate<KC_HID, false>(sm, slot, &refusal);
                         ok = executed > 0;
                         slot += ok ? executed - 1 : 0;
                         break;
