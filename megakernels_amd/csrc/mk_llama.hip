@@ -68,7 +68,8 @@ constexpr int kHotRows = 4;         // barrier rows 2..5 are sharded
 constexpr int kOutRows = 2048;      // rows staged in LDS between matvec and epilogue
 constexpr int kMaxK = 4096;         // longest activation vector handed through LDS
 constexpr int kScoreCap = 4096;     // tokens per attention partition (LDS score buffer)
-constexpr int kQueueSlots = 256;    // longest instruction queue per worker (kept in LDS)
+constexpr int kQueueSlots = 192;    // longest instruction queue per worker (kept in LDS)
+constexpr int kParkBytes = kConsumerWaves * 4096;  // one more parked row per wave, outside the score buffer
 constexpr int kMaxHeadDim = 128;
 constexpr int kGqa = 4;             // query heads per KV head handled by one attention instruction
 constexpr int kStatusInts = 16;
@@ -105,6 +106,9 @@ constexpr int rows_in_flight(int wanted) { return KC <= 4 ? wanted : (wanted < 2
 #endif
 #ifndef MK_PARK_UPGATE
 #define MK_PARK_UPGATE 1            // long-waiting O-proj + up/gate workers park up/gate's last rows in LDS
+#endif
+#ifndef MK_PARK_DOWN
+#define MK_PARK_DOWN 1              // ... and the last row per wave of the down projection that follows
 #endif
 #ifndef MK_POLL_SLEEP
 #define MK_POLL_SLEEP 10            // units of 64 clocks between two looks at a dependency
@@ -162,6 +166,8 @@ struct Smem {
     alignas(16) float wave_l[kConsumerWaves][kGqa];
     alignas(16) float wave_o[kConsumerWaves][kGqa][kMaxHeadDim];
     alignas(16) float scores[kScoreCap][kGqa];  // attention: one partition's scores, then probabilities
+    alignas(16) unsigned char park[kParkBytes];  // a weight row per wave parked for a later instruction
+    int parked_slot;                               // the instruction whose last row per wave lies in `park`, or -1
     int queue[kQueueSlots][MK_INSTRUCTION_WORDS];  // this worker's instructions, fetched once
 };
 static_assert(offsetof(Smem, x) % 16 == 0 && offsetof(Smem, wave_max) % 16 == 0 && offsetof(Smem, wave_l) % 16 == 0 &&
@@ -1180,8 +1186,8 @@ __device__ __forceinline__ void park_rows(const Ctx &c, MK_LDS unsigned char *sl
 
 // One instruction, its first Map::size rows already requested into the listed buffers: wait for the
 // activation vector, stream the rows (Map::size in flight), leave the results in LDS, and wait until
-// the controller has sent them.  PARKED > 0: the instruction has at most Map::size + PARKED rows per
-// wave and those beyond the buffers were parked in `slice` on entry, so nothing is requested here.
+// the controller has sent them.  PARKED > 0: the wave's last PARKED rows were parked in `slice` by an
+// earlier request and are taken from there; the rows before them stream as usual.
 template <int KC, class Map, int NBUF, int PARKED = 0>
 __device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&pool)[NBUF][KC], const MatvecDesc &d, int mine,
                                              MK_LDS const unsigned char *slice = nullptr) {
@@ -1195,15 +1201,17 @@ __device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&pool)[NBUF][K
         const float y = mkm::round_bf16(dot_row<KC>(src, x));
         if (c.lane == 0) c.sm->out[c.wave + i * kConsumerWaves] = y;
     };
+    const int parked_first = mine > PARKED ? mine - PARKED : 0;  // rows from here on are in LDS
+    const int streamed = PARKED > 0 ? parked_first : mine;
     int base = 0;
     // rounds that are followed by more rows: every row of the round exists, every buffer is refilled
-    for (; PARKED == 0 && base + PF < mine; base += PF) {
+    for (; base + PF < streamed; base += PF) {
 #pragma unroll
         for (int s = 0; s < PF; s++) {
             consume(pool[Map::at(s)], base + s);
             compiler_fence();
             const int i = base + s + PF;
-            load_row<KC>(pool[Map::at(s)], matvec_row(d, c.wave + i * kConsumerWaves), i < mine, c.lane);
+            load_row<KC>(pool[Map::at(s)], matvec_row(d, c.wave + i * kConsumerWaves), i < streamed, c.lane);
             compiler_fence();
         }
     }
@@ -1211,19 +1219,19 @@ __device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&pool)[NBUF][K
     // last round: nothing left to request
 #pragma unroll
     for (int s = 0; s < PF; s++)
-        if (base + s < mine) consume(pool[Map::at(s)], base + s);
+        if (base + s < streamed) consume(pool[Map::at(s)], base + s);
     if constexpr (PARKED > 0) {
         wait_stores();  // the parked rows were requested long ago; this makes their arrival in LDS certain
 #pragma unroll
         for (int r = 0; r < PARKED; r++)
-            if (PF + r < mine) {
+            if (parked_first + r < mine) {
                 uint4 row[KC];
 #pragma unroll
                 for (int j = 0; j < KC; j++) {
                     const u32x4 v = *(const MK_LDS u32x4 *)(slice + r * (KC * 1024) + j * 1024 + c.lane * 16);
                     row[j] = uint4{v.x, v.y, v.z, v.w};
                 }
-                consume(row, PF + r);
+                consume(row, parked_first + r);
             }
     }
     trace_consumer(c, 23);
@@ -1257,7 +1265,7 @@ template <> struct FirstBuffers<5> { typedef BufMap<0, 1, 2, 3, 4> type; };
 template <> struct FirstBuffers<6> { typedef BufMap<0, 1, 2, 3, 4, 5> type; };
 
 // One matvec instruction (opcode OP, row width KC chunks).
-template <int OP, int KC>
+template <int OP, int KC, int PARKED = 0>
 static __device__ __noinline__ bool op_matvec(SmemPtr lds, int slot, int *refusal) {
     constexpr int PF = rows_in_flight<KC>(pf_of(OP));
     typedef typename FirstBuffers<PF>::type Map;
@@ -1269,9 +1277,9 @@ static __device__ __noinline__ bool op_matvec(SmemPtr lds, int slot, int *refusa
     uint4 pool[PF][KC];
     wg_barrier();  // entry: the controller's first requests are out
     trace_consumer(c, 20);
-    request_rows<KC, Map>(c, pool, d, 0, mine);
+    request_rows<KC, Map>(c, pool, d, 0, mine > PARKED ? mine - PARKED : 0);
     trace_consumer(c, 21);
-    const bool ok = consumer_run<KC, Map>(c, pool, d, mine);
+    const bool ok = consumer_run<KC, Map, PF, PARKED>(c, pool, d, mine, (MK_LDS const unsigned char *)lds->park + c.wave * (KC * 1024));
     trace_consumer_flush(c, 20, 25);
     return ok;
 }
@@ -1314,14 +1322,25 @@ static __device__ __noinline__ int op_oproj_upgate(SmemPtr lds, int slot, int *r
     if (!pair) dsu = dso;  // never fetched: the requests below become no-ops
     const int mine_o = rows_of_wave(dso.ntasks, co.wave);
     const int mine_u = pair ? rows_of_wave(dsu.ntasks, co.wave) : 0;
+    const int stream_u = mine_u > kParked ? mine_u - kParked : 0;  // up/gate rows that go through the buffers
     uint4 pool[NBUF][KC];
     wg_barrier();  // entry of O-proj: the controller's first requests are out
     request_rows<KC, MapO>(co, pool, dso, 0, mine_o);
-    request_rows<KC, MapU0>(co, pool, dsu, 0, mine_u, pair);
+    request_rows<KC, MapU0>(co, pool, dsu, 0, stream_u, pair);
     MK_LDS unsigned char *slice = (MK_LDS unsigned char *)&lds->scores[0][0] + co.wave * (kParked * KC * 1024);
-    if constexpr (PARK) park_rows<KC, kParked>(co, slice, dsu, MapU::size, mine_u, pair);
+    if constexpr (PARK) {
+        park_rows<KC, kParked>(co, slice, dsu, mine_u > kParked ? mine_u - kParked : 0, mine_u, pair);
+        // and the last row per wave of a down projection that follows directly
+        MatvecDesc dsd;
+        const bool down_next = MK_PARK_DOWN && KC * 1024 * kConsumerWaves <= kParkBytes && slot + 2 < uni(lds->args.num_slots) &&
+                               uni(lds->queue[slot + 2][0]) == 6 && describe_matvec(lds, slot + 2, dsd);
+        if (!down_next) dsd = dso;
+        const int mine_d = down_next ? rows_of_wave(dsd.ntasks, co.wave) : 0;
+        park_rows<KC, 1>(co, (MK_LDS unsigned char *)lds->park + co.wave * (KC * 1024), dsd, mine_d > 0 ? mine_d - 1 : 0, mine_d, down_next);
+        if (co.lane == 0 && co.wave == 0) lds->parked_slot = down_next ? slot + 2 : -1;
+    }
     if (!consumer_run<KC, MapO>(co, pool, dso, mine_o)) return 0;
-    request_rows<KC, MapU1>(co, pool, dsu, MapU0::size, mine_u, pair);
+    request_rows<KC, MapU1>(co, pool, dsu, MapU0::size, stream_u, pair);
     if (!pair) return 1;
     wg_barrier();  // entry of up/gate: its first requests went out long ago
     return consumer_run<KC, MapU, NBUF, kParked>(cu, pool, dsu, mine_u, slice) ? 2 : 0;
@@ -1809,6 +1828,7 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
     if (tid == 0) {
         sm->abort = 0;
         sm->last_flag = 0;
+        sm->parked_slot = -1;
         sm->t_launch = wall_clock64();
         // the token whose embedding row starts the step (written by the previous launch or the host)
         int token = -1;
@@ -1883,7 +1903,15 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
                 ok = op_matvec<4, KC_RED>(sm, slot, &refusal);
                 break;
             case 5: ok = op_matvec<5, KC_HID>(sm, slot, &refusal); break;
-            case 6: ok = op_matvec<6, KC_RED>(sm, slot, &refusal); break;
+            case 6:
+            if constexpr (KC_HID == KC_RED && MK_PAIR_OPROJ_UPGATE && MK_PARK_UPGATE && MK_PARK_DOWN) {
+                if (sm->parked_slot == slot) {
+                    ok = op_matvec<6, KC_RED, 1>(sm, slot, &refusal);
+                    break;
+                }
+            }
+            ok = op_matvec<6, KC_RED>(sm, slot, &refusal);
+            break;
             case 7: ok = op_lm_head<KC_HID>(sm, slot, &refusal); break;
             default: ok = bail(make_ctx(sm, slot, opcode), MK_STATUS_BAD_OPCODE, &refusal);  // reference: trap, include/util.cuh:38
             }
@@ -2036,7 +2064,10 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
             }
         }
         if (!more) break;
-        if (tid == 0) sm->args.pos_id = a.pos_id + step + 1;
+        if (tid == 0) {
+            sm->args.pos_id = a.pos_id + step + 1;
+            sm->parked_slot = -1;
+        }
         wg_barrier();
         if (sm->abort) break;
     }
