@@ -1889,9 +1889,11 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
             case 4:
                 if constexpr (KC_HID == KC_RED && MK_PAIR_OPROJ_UPGATE) {
                     if (slot + 1 < a.num_slots && sm->queue[slot + 1][0] == 5) {
-                        // rows can be parked when the wait is long (no attention just before) and the
-                        // up/gate instruction is small enough (two list entries: eight rows per wave)
-                        const bool park = MK_PARK_UPGATE && (slot == 0 || sm->queue[slot - 1][0] != 2) &&
+                        // rows can be parked when the wait is long (no attention just before, and a
+                        // partition merge between attention and O-proj: with a single partition per head
+                        // the wait is too short for it to pay) and the up/gate instruction is small
+                        // enough (two list entries: eight rows per wave)
+                        const bool park = MK_PARK_UPGATE && !a.skip_attn_reduction && (slot == 0 || sm->queue[slot - 1][0] != 2) &&
                                           sm->queue[slot + 1][2] >= 0 && sm->queue[slot + 1][2] <= 2;
                         const int executed = park ? op_oproj_upgate<KC_HID, true>(sm, slot, &refusal)
                                                   : op_oproj_upgate<KC_HID, false>(sm, slot, &refusal);
