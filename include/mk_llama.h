@@ -27,14 +27,32 @@ extern "C" {
 #define MK_TIMING_SLOTS 128       /* megakernels/scheduler.py:14, include/config.cuh:18 */
 #define MK_BARRIER_ROWS 10        /* megakernels/demos/latency/scheduler.py:53-61 */
 
-/* args.flags: record per-instruction timings into `timings` (slot 0 start, 1 dependency ready,
- * 2 matvec done, 3 end - ticks of the 100 MHz wall clock since the workgroup started; slot 4 opcode).
- * Counterpart of the reference's compile-time TIMING_RECORD_ENABLED (include/config.cuh:46). */
+/* args.flags: record per-instruction timings into `timings[worker, slot, :]` - ticks of the 100 MHz
+ * wall clock since the workgroup started, written by the workgroup's controller wave.  Counterpart
+ * of the reference's compile-time TIMING_RECORD_ENABLED (include/config.cuh:46); the word indices
+ * are MK_TIMING_* below. */
 #define MK_FLAG_TIMINGS 1u
 /* args.flags: leave `barriers` all zero after the launch instead of holding the VM's counts, so that
  * the next launch needs no reset (the reference's loop refills the tensor before every launch,
  * megakernels/generators.py:127-128). */
 #define MK_FLAG_RESET_BARRIERS 2u
+
+/* Words of one instruction's timing record.  Words 0 and 4 are the reference's
+ * TEVENT_CONTROLLER_START and TEVENT_CONTROLLER_END (include/util.cuh:215-219).  Words 1-3 are
+ * instruction fetch done, page allocation done and semaphore set-up in the reference - stages this
+ * kernel does not have (the queue is in LDS, there are no pages or semaphores) - and hold the stages
+ * it has instead.  The reference's loader / consumer / storer events (words 5-54,
+ * include/util.cuh:220-239) are not written by the kernel; megakernels_amd/scripts/timeline.py
+ * fills them from these five on the host for tools that read the reference's layout.
+ * For every executed instruction START <= DEPENDENCY_READY <= INPUT_READY <= COMPUTE_DONE <= END. */
+enum {
+    MK_TIMING_START = 0,            /* the controller wave took the instruction */
+    MK_TIMING_DEPENDENCY_READY = 1, /* the barrier counters it waits for reached their targets */
+    MK_TIMING_INPUT_READY = 2,      /* activation vector normalised and handed to the consumer waves */
+    MK_TIMING_COMPUTE_DONE = 3,     /* all rows of the instruction computed */
+    MK_TIMING_END = 4,              /* results stored and signalled */
+    MK_TIMING_OPCODE = 5            /* the instruction's opcode, not a time */
+};
 
 /* Status codes written by the kernel into the workspace and returned by
  * mk_llama_read_status(). */

@@ -428,7 +428,10 @@ __device__ __forceinline__ long long spin_ticks(const Ctx &c) {
 // Timing slots written per instruction by the controller when MK_FLAG_TIMINGS is set (ticks of
 // the 100 MHz wall clock since the workgroup started; counterpart of the reference's timing
 // events, include/util.cuh:215-246).
-enum { kEvStart = 0, kEvDepReady = 1, kEvInputReady = 2, kEvComputeDone = 3, kEvEnd = 4, kEvOpcode = 5 };
+enum {
+    kEvStart = MK_TIMING_START, kEvDepReady = MK_TIMING_DEPENDENCY_READY, kEvInputReady = MK_TIMING_INPUT_READY,
+    kEvComputeDone = MK_TIMING_COMPUTE_DONE, kEvEnd = MK_TIMING_END, kEvOpcode = MK_TIMING_OPCODE
+};
 
 __device__ __forceinline__ void trace_event(const Ctx &c, int slot) {
     if (c.trace && c.controller && c.lane == 0) st_plain_i32(c.trace + slot, (int)(wall_clock64() - c.sm->t_launch));
@@ -2139,10 +2142,12 @@ int mk_llama_query(int what) {
     }
 }
 
-int mk_llama_launch(const mk_llama_args *args, void *hip_stream) {
-    g_error[0] = 0;
-    if (!args) return fail(-1, "null arguments");
-    const mk_llama_args &a = *args;
+}  // extern "C"
+
+namespace {
+
+// validate the arguments against what the kernel assumes and pick the kernel instance
+int validate(const mk_llama_args &a, KernelFn *kernel) {
     const void *required[] = {a.barriers, a.instructions, a.qkv_weights, a.attn_norm_weights, a.o_weights,
                               a.mlp_norm_weights, a.up_weights, a.gate_weights, a.down_weights,
                               a.lm_head_norm_weights, a.lm_head_weights, a.k_cache, a.v_cache, a.rope_cos,
@@ -2204,22 +2209,60 @@ int mk_llama_launch(const mk_llama_args *args, void *hip_stream) {
     if (a.num_workers > cus)
         return fail(-7, "schedule has %d workers but the device has %d compute units", a.num_workers, cus);
 
-    static thread_local KernelFn configured[8] = {};
-    bool seen = false;
-    for (KernelFn f : configured) seen |= f == fn;
-    if (!seen) {
+    *kernel = fn;
+    return 0;
+}
+
+int launch_kernel(KernelFn fn, const mk_llama_args &a, void *hip_stream) {
+    // Per kernel instance, once: allow the LDS request, and ask the runtime how many workgroups of
+    // this shape the device holds at once.  Every barrier wait assumes that all workers are running
+    // (the reference: one block per SM by __launch_bounds__(NUM_THREADS, 1) and grid = SM count,
+    // include/megakernel.cuh:166-171), so a grid that cannot be resident as a whole is refused here
+    // rather than found out by the waits' time limit.
+    struct Configured {
+        KernelFn fn;
+        int device, resident;
+    };
+    static thread_local Configured configured[16] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return fail(-7, "cannot query the device");
+    int resident = -1;
+    for (const Configured &k : configured)
+        if (k.fn == fn && k.device == dev) resident = k.resident;
+    if (resident < 0) {
         hipError_t e = hipFuncSetAttribute((const void *)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Smem));
         if (e != hipSuccess) return fail(-8, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-        for (KernelFn &f : configured)
-            if (!f) {
-                f = fn;
+        int per_cu = 0, cus = 0;
+        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void *)fn, kThreads, sizeof(Smem));
+        if (e != hipSuccess) return fail(-8, "hipOccupancyMaxActiveBlocksPerMultiprocessor: %s", hipGetErrorString(e));
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+            return fail(-7, "cannot query the device");
+        resident = per_cu * cus;
+        for (Configured &k : configured)
+            if (!k.fn) {
+                k = Configured{fn, dev, resident};
                 break;
             }
     }
+    if (a.num_workers > resident)
+        return fail(-7, "schedule has %d workers but only %d workgroups of this kernel can be resident at once", a.num_workers,
+                    resident);
     hipLaunchKernelGGL(fn, dim3(a.num_workers), dim3(kThreads), sizeof(Smem), (hipStream_t)hip_stream, a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(-9, "kernel launch: %s", hipGetErrorString(e));
     return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mk_llama_launch(const mk_llama_args *args, void *hip_stream) {
+    g_error[0] = 0;
+    if (!args) return fail(-1, "null arguments");
+    KernelFn fn = nullptr;
+    if (const int rc = validate(*args, &fn)) return rc;
+    return launch_kernel(fn, *args, hip_stream);
 }
 
 int mk_llama_selftest_bf16(uint64_t *mismatches_out) {
