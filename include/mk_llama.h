@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define MK_LLAMA_ABI_VERSION 3
+#define MK_LLAMA_ABI_VERSION 4
 #define MK_INSTRUCTION_WORDS 32   /* megakernels/scheduler.py:13, include/config.cuh:14 */
 #define MK_TIMING_SLOTS 128       /* megakernels/scheduler.py:14, include/config.cuh:18 */
 #define MK_BARRIER_ROWS 10        /* megakernels/demos/latency/scheduler.py:53-61 */
@@ -139,6 +139,18 @@ uint64_t mk_llama_workspace_bytes(int32_t num_layers, int32_t hidden_size, int32
  * mk_llama_last_error().  Replaces the `mk_llama(...)` call of
  * megakernels/demos/latency/mk.py:15-49. */
 int mk_llama_launch(const mk_llama_args *args, void *hip_stream);
+
+/* The same launch for callers that cannot allocate device memory and have no workspace to bring:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No
+ * counterpart in the reference.  `args->workspace` and `args->workspace_bytes` are ignored; the
+ * workspace is an array inside the library (2 MiB per GPU, held until the process ends), which is
+ * enough for every shape the kernel has an instance for (1B: 250 KB, 8B with 32 layers: 950 KB).
+ * Shapes that need more are refused with -6 and a message.  The call allocates nothing: it zeroes
+ * the part of the array it is going to use with a small kernel on `hip_stream`, then launches as
+ * mk_llama_launch does.  `*scratch_out` (may be NULL) receives the array's device address, which is
+ * what mk_llama_read_status() takes as `workspace`.  All calls on one GPU share the array: two
+ * launches that overlap in time on one GPU (different streams, different threads) race. */
+int mk_llama_launch_static(const mk_llama_args *args, void *hip_stream, void **scratch_out);
 
 /* Synchronises `hip_stream` and copies the 4-word status block
  * {code, worker, slot, opcode} of the workspace to the host.  A non-zero code

@@ -46,6 +46,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <type_traits>
 
 #include "../../include/mk_llama.h"
@@ -2093,6 +2094,21 @@ __global__ void bf16_convert_sweep_kernel(unsigned long long *mismatches) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// Workspace for callers that cannot allocate (mk_llama_launch_static): one array per GPU, held from
+// the moment the library is loaded on that GPU until the process ends.  In host code the array's
+// name is only a handle for hipGetSymbolAddress; kernels get the address that call returns.
+// ---------------------------------------------------------------------------------------------
+constexpr size_t kStaticScratchBytes = 2u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Zeroes `count` 16-byte units.  A kernel rather than a memset: the launch may be recorded into a
+// graph by the caller, where memset nodes are best avoided.
+__global__ void scratch_clear_kernel(uint4 *dst, size_t count) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride) dst[i] = make_uint4(0, 0, 0, 0);
+}
+
+// ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
 thread_local char g_error[512] = "";
@@ -2253,6 +2269,26 @@ int launch_kernel(KernelFn fn, const mk_llama_args &a, void *hip_stream) {
     return 0;
 }
 
+// device address of this GPU's copy of `scratch`, looked up once per device
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(void **out) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return fail(-7, "cannot query the device");
+    if (dev < 0 || dev >= kMaxDevices) return fail(-7, "device index %d beyond the %d the library keeps scratch addresses for", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) return fail(-8, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -2263,6 +2299,33 @@ int mk_llama_launch(const mk_llama_args *args, void *hip_stream) {
     KernelFn fn = nullptr;
     if (const int rc = validate(*args, &fn)) return rc;
     return launch_kernel(fn, *args, hip_stream);
+}
+
+int mk_llama_launch_static(const mk_llama_args *args, void *hip_stream, void **scratch_out) {
+    g_error[0] = 0;
+    if (!args) return fail(-1, "null arguments");
+    mk_llama_args a = *args;
+    const uint64_t need = mk_llama_workspace_bytes(a.num_layers, a.hidden_size, a.intermediate_size, a.matvec_reduction_size);
+    if (need == 0) return fail(-3, "empty model or schedule");
+    if (need > kStaticScratchBytes)
+        return fail(-6, "these shapes need %llu bytes of workspace, the library's static scratch holds %llu: use mk_llama_launch with a caller-owned workspace",
+                    (unsigned long long)need, (unsigned long long)kStaticScratchBytes);
+    void *ptr = nullptr;
+    if (const int rc = static_scratch(&ptr)) return rc;
+    a.workspace = ptr;
+    a.workspace_bytes = kStaticScratchBytes;
+    KernelFn fn = nullptr;
+    if (const int rc = validate(a, &fn)) return rc;
+    if (scratch_out) *scratch_out = ptr;
+    // The array keeps whatever the last call left: counters are back at zero after a launch that
+    // completed, but the residual partial sums of other shapes may lie where this call's counters
+    // go, and a launch that gave up leaves its status behind.  Everything this call uses starts at zero.
+    const size_t units = (size_t)((need + 15) / 16);
+    hipLaunchKernelGGL(scratch_clear_kernel, dim3((unsigned)((units + 255) / 256)), dim3(256), 0, (hipStream_t)hip_stream,
+                       static_cast<uint4 *>(ptr), units);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(-9, "scratch clear launch: %s", hipGetErrorString(e));
+    return launch_kernel(fn, a, hip_stream);
 }
 
 int mk_llama_selftest_bf16(uint64_t *mismatches_out) {

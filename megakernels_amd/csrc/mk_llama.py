@@ -57,6 +57,10 @@ _workspaces: dict[tuple, torch.Tensor] = {}
 spin_limit_us = 0
 # set to True to have every launch fill the `timings` tensor (see MK_FLAG_TIMINGS in mk_llama.h)
 record_timings = False
+# set to True to launch through mk_llama_launch_static: the workspace is then the library's own
+# per-GPU array and this module allocates nothing for a launch
+static_scratch = False
+_static_scratch_ptrs: dict[int, int] = {}
 
 
 def load_library():
@@ -69,6 +73,8 @@ def load_library():
         lib = ctypes.CDLL(str(LIBRARY))
         lib.mk_llama_launch.argtypes = [ctypes.POINTER(MkLlamaArgs), _P]
         lib.mk_llama_launch.restype = ctypes.c_int
+        lib.mk_llama_launch_static.argtypes = [ctypes.POINTER(MkLlamaArgs), _P, ctypes.POINTER(_P)]
+        lib.mk_llama_launch_static.restype = ctypes.c_int
         lib.mk_llama_workspace_bytes.argtypes = [_I, _I, _I, _I]
         lib.mk_llama_workspace_bytes.restype = ctypes.c_uint64
         lib.mk_llama_read_status.argtypes = [_P, _P, ctypes.POINTER(_I * 4)]
@@ -202,9 +208,10 @@ def mk_llama(
     a.rope_positions = rope_cos.shape[0]
     a.matvec_reduction_size = reduction
     a.attn_reduction_size = 4
-    ws = _workspace(barriers.device, num_layers, hidden, inter, reduction)
-    a.workspace = ws.data_ptr()
-    a.workspace_bytes = ws.numel() * 4
+    if not static_scratch:
+        ws = _workspace(barriers.device, num_layers, hidden, inter, reduction)
+        a.workspace = ws.data_ptr()
+        a.workspace_bytes = ws.numel() * 4
     a.spin_limit_us = int(spin_limit_us)
     a.flags = (1 if (record_timings and timings is not None) else 0) | (2 if reset_barriers else 0)
     if token_in is not None:
@@ -221,7 +228,14 @@ def mk_llama(
 
     if stream is None:
         stream = torch.cuda.current_stream(barriers.device)
-    rc = lib.mk_llama_launch(ctypes.byref(a), ctypes.c_void_p(stream.cuda_stream))
+    if static_scratch:
+        with torch.cuda.device(barriers.device):
+            where = _P()
+            rc = lib.mk_llama_launch_static(ctypes.byref(a), ctypes.c_void_p(stream.cuda_stream), ctypes.byref(where))
+        if rc == 0:
+            _static_scratch_ptrs[barriers.device.index] = where.value
+    else:
+        rc = lib.mk_llama_launch(ctypes.byref(a), ctypes.c_void_p(stream.cuda_stream))
     if rc != 0:
         raise RuntimeError(f"mk_llama_launch failed ({rc}): {lib.mk_llama_last_error().decode()}")
 
@@ -239,17 +253,27 @@ def read_status(device=None, stream=None):
     device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
     out = (_I * 4)()
     result = (0, 0, 0, 0)
+    if stream is None:
+        stream = torch.cuda.current_stream(device)
     for key, ws in _workspaces.items():
         if key[0] != device.index:
             continue
-        if stream is None:
-            stream = torch.cuda.current_stream(device)
         rc = lib.mk_llama_read_status(ctypes.c_void_p(ws.data_ptr()), ctypes.c_void_p(stream.cuda_stream), ctypes.byref(out))
         if rc != 0:
             raise RuntimeError(f"mk_llama_read_status failed: {lib.mk_llama_last_error().decode()}")
         if out[0] != 0:
             result = tuple(out)
             ws.zero_()
+    # the library's own array (launches with static_scratch): every such launch clears what it uses
+    # first, so a recorded failure needs no clean-up here
+    where = _static_scratch_ptrs.get(device.index)
+    if where and result[0] == 0:
+        rc = lib.mk_llama_read_status(ctypes.c_void_p(where), ctypes.c_void_p(stream.cuda_stream), ctypes.byref(out))
+        if rc != 0:
+            raise RuntimeError(f"mk_llama_read_status failed: {lib.mk_llama_last_error().decode()}")
+        if out[0] != 0:
+            result = tuple(out)
+            del _static_scratch_ptrs[device.index]
     return result
 
 

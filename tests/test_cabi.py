@@ -30,7 +30,7 @@ def load():
 
 
 def test_header_declares_the_expected_entry_points():
-    assert declared_functions() == ["mk_llama_last_error", "mk_llama_launch", "mk_llama_query",
+    assert declared_functions() == ["mk_llama_last_error", "mk_llama_launch", "mk_llama_launch_static", "mk_llama_query",
                                     "mk_llama_read_status", "mk_llama_selftest_bf16", "mk_llama_workspace_bytes"]
 
 
@@ -51,7 +51,7 @@ def test_workspace_size_and_static_queries():
     assert small == 4 * (32 + 4 * 16 * 16 * 4 + 128 + 128 + 2 * 1024 + 4 * 2048 + 16 * 2 * 48 * 32)
     assert big > small and big < (1 << 20)
     assert lib.mk_llama_workspace_bytes(0, 2048, 8192, 2048) == 0
-    assert lib.mk_llama_query(3) == 3                      # ABI version
+    assert lib.mk_llama_query(3) == 4                      # ABI version
     assert lib.mk_llama_query(2) == 576                    # 8 consumer waves + 1 controller wave
     assert 80 * 1024 < lib.mk_llama_query(1) <= 160 * 1024  # one workgroup per CU, within gfx950's LDS
     assert lib.mk_llama_query(4) >= 2048
@@ -70,6 +70,25 @@ def test_launch_refuses_null_arguments_without_touching_a_gpu():
     args = mk_llama.MkLlamaArgs()  # all pointers null
     assert lib.mk_llama_launch(ctypes.byref(args), None) == -2
     assert b"null device pointer" in lib.mk_llama_last_error()
+
+
+def test_static_scratch_launch_refuses_shapes_beyond_its_array_before_touching_a_gpu():
+    lib = load()
+    lib.mk_llama_last_error.restype = ctypes.c_char_p
+    lib.mk_llama_workspace_bytes.restype = ctypes.c_uint64
+    lib.mk_llama_workspace_bytes.argtypes = [ctypes.c_int32] * 4
+    lib.mk_llama_launch_static.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    assert lib.mk_llama_launch_static(None, None, None) == -1
+    import sys
+    sys.path.insert(0, str(LIB.parent))
+    import mk_llama
+    args = mk_llama.MkLlamaArgs()
+    args.num_layers, args.hidden_size, args.intermediate_size, args.matvec_reduction_size = 512, 4096, 14336, 2048
+    assert lib.mk_llama_workspace_bytes(512, 4096, 14336, 2048) > (2 << 20)
+    assert lib.mk_llama_launch_static(ctypes.byref(args), None, None) == -6
+    assert b"static scratch" in lib.mk_llama_last_error()
+    # every shape the kernel has an instance for fits
+    assert lib.mk_llama_workspace_bytes(32, 4096, 14336, 2048) <= (2 << 20)
 
 
 def test_python_args_struct_matches_the_header():
