@@ -286,30 +286,38 @@ class LlamaForCausalLM:
         device: DeviceType = "cpu",
         dtype: torch.dtype = torch.bfloat16,
         std: float = 0.02,
+        draw_device: DeviceType | None = None,
     ) -> "LlamaForCausalLM":
         """Random-initialised model: every matrix is drawn ``N(0, std)`` in fp32
         from a CPU generator seeded with ``seed`` and cast to ``dtype``; norm
         weights are one.  Draw order: embedding; per layer q, k, v, o, up, gate,
         down; then the LM head when it is not tied to the embedding.  The same
         seed yields the same bits on every host, so a CPU checker and the GPU
-        run can be fed identical weights."""
+        run can be fed identical weights.  ``draw_device``: draw with that
+        device's generator instead (a GPU fills the 8B architecture in seconds
+        where the CPU generator takes minutes; the bits then belong to that
+        generator, and a CPU twin is made with ``.to("cpu")``)."""
         extra_config = extra_config or ExtraModelConfig(interleave_rope=True)
-        gen = torch.Generator(device="cpu").manual_seed(seed)
+        draw_device = torch.device(draw_device or "cpu")
+        gen = torch.Generator(device=draw_device).manual_seed(seed)
         c = config
         H, KVH, D = c.num_attention_heads, c.num_key_value_heads, c.head_dim
         L, hid, inter = c.num_hidden_layers, c.hidden_size, c.intermediate_size
 
         def draw(rows, cols):
-            return torch.empty(rows, cols, dtype=torch.float32).normal_(0.0, std, generator=gen).to(dtype)
+            return torch.empty(rows, cols, dtype=torch.float32, device=draw_device).normal_(0.0, std, generator=gen).to(dtype)
+
+        def stack(*shape):
+            return torch.empty(*shape, dtype=dtype, device=draw_device)
 
         embed = draw(c.vocab_size, hid)
-        qkv = torch.empty(L, (H + 2 * KVH) * D, hid, dtype=dtype)
-        o = torch.empty(L, hid, H * D, dtype=dtype)
-        up = torch.empty(L, inter, hid, dtype=dtype)
-        gate = torch.empty(L, inter, hid, dtype=dtype)
-        down = torch.empty(L, hid, inter, dtype=dtype)
-        q_perm = interleave_permutation(D, H)
-        k_perm = interleave_permutation(D, KVH)
+        qkv = stack(L, (H + 2 * KVH) * D, hid)
+        o = stack(L, hid, H * D)
+        up = stack(L, inter, hid)
+        gate = stack(L, inter, hid)
+        down = stack(L, hid, inter)
+        q_perm = interleave_permutation(D, H).to(draw_device)
+        k_perm = interleave_permutation(D, KVH).to(draw_device)
         for layer in range(L):
             q, k, v = draw(H * D, hid), draw(KVH * D, hid), draw(KVH * D, hid)
             if extra_config.interleave_rope:

@@ -56,6 +56,28 @@ def fill_kv(model, upto: int, seed=2, poison=True):
             cache[:, :, upto:] = 0
 
 
+def make_model_pair(cfg, max_len, seed=0, device="cuda:0"):
+    """(CPU model, GPU model) with identical weights drawn by the GPU's generator: the full-size
+    architectures take seconds this way and minutes with the CPU generator."""
+    model_gpu = LlamaForCausalLM.from_random(
+        cfg, ExtraModelConfig(interleave_rope=True, max_len_override=max_len), seed=seed, device=device, draw_device=device
+    )
+    return model_gpu.to("cpu"), model_gpu
+
+
+def fill_kv_pair(model_cpu, model_gpu, upto: int, seed=2):
+    """fill_kv for a model pair: drawn on the GPU, copied to the CPU twin.  Seeded N(0,1) for
+    positions [0, upto), N(0,100) beyond."""
+    gen = torch.Generator(device=model_gpu.device).manual_seed(seed)
+    for dst, twin in zip(model_gpu.stacked_kv_cache, model_cpu.stacked_kv_cache):
+        # layer by layer: the fp32 draw of a whole 32k-position cache is a multiple of the cache itself
+        for layer in range(dst.shape[0]):
+            rows = torch.randn(dst.shape[1:], generator=gen, device=dst.device)
+            rows[:, upto:] *= 100
+            dst[layer].copy_(rows)
+        twin.copy_(dst)
+
+
 def build_schedule(model, workers, partitions=1, sched="rr", stop_after_op=None, layer_limit=None):
     set_sm_count_override(workers)
     schedule = LatencyScheduleBuilder.build(
@@ -66,12 +88,14 @@ def build_schedule(model, workers, partitions=1, sched="rr", stop_after_op=None,
     return schedule
 
 
-def mirror_to_gpu(model_cpu, schedule_cpu, device="cuda:0"):
+def mirror_to_gpu(model_cpu, schedule_cpu, device="cuda:0", model_gpu=None):
     """GPU twin of a CPU model + schedule: same weights, same KV contents, same
-    instruction tensor, fresh activation buffers holding the same values."""
-    model_gpu = model_cpu.to(device)
-    for dst, src in zip(model_gpu.stacked_kv_cache, model_cpu.stacked_kv_cache):
-        dst.copy_(src)
+    instruction tensor, fresh activation buffers holding the same values.
+    ``model_gpu``: an existing twin of the model (weights and KV already equal)."""
+    if model_gpu is None:
+        model_gpu = model_cpu.to(device)
+        for dst, src in zip(model_gpu.stacked_kv_cache, model_cpu.stacked_kv_cache):
+            dst.copy_(src)
     workers = schedule_cpu.globs.instructions.shape[0]
     set_sm_count_override(workers)
     gcpu = schedule_cpu.globs
