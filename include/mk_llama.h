@@ -27,8 +27,10 @@ extern "C" {
 #define MK_TIMING_SLOTS 128       /* megakernels/scheduler.py:14, include/config.cuh:18 */
 #define MK_BARRIER_ROWS 10        /* megakernels/demos/latency/scheduler.py:53-61 */
 
-/* args.flags: record per-instruction timings into `timings[worker, slot, :]` - ticks of the 100 MHz
- * wall clock since the workgroup started, written by the workgroup's controller wave.  Counterpart
+/* args.flags: record per-instruction timings into `timings[worker, slot, :]` - the low 32 bits of
+ * the device's 100 MHz wall clock (one clock for all compute units, so records of different workers
+ * compare directly; subtract the smallest to get times since the first workgroup started), written
+ * by the workgroup's controller wave.  Counterpart
  * of the reference's compile-time TIMING_RECORD_ENABLED (include/config.cuh:46); the word indices
  * are MK_TIMING_* below. */
 #define MK_FLAG_TIMINGS 1u

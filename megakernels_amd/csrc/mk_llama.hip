@@ -151,11 +151,31 @@ __host__ __device__ inline WsLayout ws_layout(int L, int hid, int inter, int R) 
 // ---------------------------------------------------------------------------------------------
 // LDS layout
 // ---------------------------------------------------------------------------------------------
+// What every instruction needs and no instruction changes: computed once per launch, read from LDS.
+struct Consts {
+    int *status, *shards, *arrive_o, *arrive_d, *argmax, *pads;  // regions of the workspace
+    float *partial;
+    int *trace_base;                // this worker's rows of `timings`, or nullptr when tracing is off
+    long long spin_ticks;           // limit of a dependency wait, in wall-clock ticks
+    int cols;                       // columns of `barriers`: query + key + value heads
+    int pad_cols;                   // padded per-head counters per (layer, row)
+    int down_jobs, o_jobs;          // arrivals that complete barrier rows 5 and 3
+};
+// A matvec instruction (opcodes 1, 4, 5, 6) decoded once per launch: where its weight rows live.
+// ntasks < 0: the instruction is malformed.
+struct alignas(16) SlotDesc {
+    uint64_t w0_base;               // buffer the rows are addressed in
+    long long gate_delta;           // opcode 5: byte distance from the up matrix to the gate matrix
+    uint32_t w0_bytes, row_bytes;
+    int ntasks, first_row;
+};
+static_assert(sizeof(SlotDesc) == 32, "two 16-byte LDS reads");
+
 struct Smem {
     int abort;                      // set once, never cleared during a launch
     int last_flag;
     int token;                      // *token_in, or -1
-    long long t_launch;             // wall clock when the workgroup started
+    Consts k;
     mk_llama_args args;             // the launch arguments, read from here by every instruction
     int flags[kOutRows / 16];       // per-block "I was the last arriver" (matvec-add)
 #ifdef MK_TRACE_CONSUMER
@@ -169,7 +189,8 @@ struct Smem {
     alignas(16) float scores[kScoreCap][kGqa];  // attention: one partition's scores, then probabilities
     alignas(16) unsigned char park[kParkBytes];  // a weight row per wave parked for a later instruction
     int parked_slot;                               // the instruction whose last row per wave lies in `park`, or -1
-    int queue[kQueueSlots][MK_INSTRUCTION_WORDS];  // this worker's instructions, fetched once
+    alignas(16) SlotDesc desc[kQueueSlots];        // the matvec instructions of the queue, decoded once
+    alignas(16) int queue[kQueueSlots][MK_INSTRUCTION_WORDS];  // this worker's instructions, fetched once
 };
 static_assert(offsetof(Smem, x) % 16 == 0 && offsetof(Smem, wave_max) % 16 == 0 && offsetof(Smem, wave_l) % 16 == 0 &&
                   offsetof(Smem, scores) % 16 == 0,
@@ -390,7 +411,6 @@ struct Ctx {
 };
 
 __device__ __forceinline__ Ctx make_ctx(SmemPtr sm, int slot, int opcode) {
-    ArgsRef a = sm->args;
     Ctx c;
     c.sm = sm;
     c.tid = (int)threadIdx.x;
@@ -400,48 +420,37 @@ __device__ __forceinline__ Ctx make_ctx(SmemPtr sm, int slot, int opcode) {
     c.worker = (int)blockIdx.x;
     c.slot = slot;
     c.opcode = opcode;
-    c.trace = nullptr;
-    if ((a.flags & MK_FLAG_TIMINGS) && a.timings)
-        c.trace = uni(a.timings) + ((size_t)c.worker * uni(a.num_slots) + slot) * MK_TIMING_SLOTS;
+    int *const rows = uni(sm->k.trace_base);
+    c.trace = rows ? rows + (size_t)slot * MK_TIMING_SLOTS : nullptr;
     return c;
 }
 
 // workspace regions
-__device__ __forceinline__ int *ws_ints(const Ctx &c) { return uni(static_cast<int *>(c.sm->args.workspace)); }
-__device__ __forceinline__ WsLayout ws_regions(const Ctx &c) {
-    ArgsRef a = c.sm->args;
-    return ws_layout(uni(a.num_layers), uni(a.hidden_size), uni(a.intermediate_size), uni(a.matvec_reduction_size));
-}
-__device__ __forceinline__ int *ws_status(const Ctx &c) { return ws_ints(c) + ws_regions(c).status; }
-__device__ __forceinline__ int *ws_shards(const Ctx &c) { return ws_ints(c) + ws_regions(c).shards; }
-__device__ __forceinline__ int *ws_arrive(const Ctx &c, bool down) {
-    const WsLayout w = ws_regions(c);
-    return ws_ints(c) + (down ? w.arrive_d : w.arrive_o);
-}
-__device__ __forceinline__ float *ws_partial(const Ctx &c) {
-    return reinterpret_cast<float *>(ws_ints(c) + ws_regions(c).partial);
-}
+__device__ __forceinline__ int *ws_status(const Ctx &c) { return uni(c.sm->k.status); }
+__device__ __forceinline__ int *ws_shards(const Ctx &c) { return uni(c.sm->k.shards); }
+__device__ __forceinline__ int *ws_arrive(const Ctx &c, bool down) { return uni(down ? c.sm->k.arrive_d : c.sm->k.arrive_o); }
+__device__ __forceinline__ float *ws_partial(const Ctx &c) { return uni(c.sm->k.partial); }
 __device__ __forceinline__ long long spin_ticks(const Ctx &c) {
-    const uint32_t us = (uint32_t)uni((int)c.sm->args.spin_limit_us);
-    return (long long)(us ? us : 2000000u) * 100;  // 100 MHz wall clock
+    const long long v = c.sm->k.spin_ticks;
+    return ((long long)uni((int)(v >> 32)) << 32) | (uint32_t)uni((int)v);
 }
 
-// Timing slots written per instruction by the controller when MK_FLAG_TIMINGS is set (ticks of
-// the 100 MHz wall clock since the workgroup started; counterpart of the reference's timing
-// events, include/util.cuh:215-246).
+// Timing slots written per instruction by the controller when MK_FLAG_TIMINGS is set (low 32 bits
+// of the device's 100 MHz wall clock, the same clock on every compute unit; counterpart of the
+// reference's timing events, include/util.cuh:215-246).
 enum {
     kEvStart = MK_TIMING_START, kEvDepReady = MK_TIMING_DEPENDENCY_READY, kEvInputReady = MK_TIMING_INPUT_READY,
     kEvComputeDone = MK_TIMING_COMPUTE_DONE, kEvEnd = MK_TIMING_END, kEvOpcode = MK_TIMING_OPCODE
 };
 
 __device__ __forceinline__ void trace_event(const Ctx &c, int slot) {
-    if (c.trace && c.controller && c.lane == 0) st_plain_i32(c.trace + slot, (int)(wall_clock64() - c.sm->t_launch));
+    if (c.trace && c.controller && c.lane == 0) st_plain_i32(c.trace + slot, (int)(uint32_t)wall_clock64());
 }
 
 // consumer-side events (wave 0, lane 0), slots 16 and up; for kernel development
 __device__ __forceinline__ void trace_consumer(const Ctx &c, int slot) {
 #ifdef MK_TRACE_CONSUMER
-    if (c.trace && c.tid == 0) c.sm->consumer_ticks[slot - 16] = (int)(wall_clock64() - c.sm->t_launch);
+    if (c.trace && c.tid == 0) c.sm->consumer_ticks[slot - 16] = (int)(uint32_t)wall_clock64();
 #endif
 }
 __device__ __forceinline__ void trace_consumer_flush(const Ctx &c, int first, int last) {
@@ -452,9 +461,7 @@ __device__ __forceinline__ void trace_consumer_flush(const Ctx &c, int first, in
 }
 
 __device__ __forceinline__ int *bar_ptr(const Ctx &c, int layer, int row, int col) {
-    ArgsRef a = c.sm->args;
-    const int cols = uni(a.num_attention_heads) + 2 * uni(a.num_kv_heads);
-    return uni(a.barriers) + ((size_t)layer * MK_BARRIER_ROWS + row) * cols + col;
+    return uni(c.sm->args.barriers) + ((size_t)layer * MK_BARRIER_ROWS + row) * uni(c.sm->k.cols) + col;
 }
 // [replica][shard][layer][row]: the shards of one counter lie in different cache lines
 // Barrier rows 0 (QKV blocks per head) and 1 (attention partitions per head) while the kernel runs.
@@ -462,8 +469,7 @@ __device__ __forceinline__ int *bar_ptr(const Ctx &c, int layer, int row, int co
 // microsecond then queue up behind each other (same-line atomics are served one at a time) and
 // the waiting side sees its own head complete late.  Here every counter has a line of its own.
 __device__ __forceinline__ int *pad_ptr(const Ctx &c, int layer, int row, int col) {
-    ArgsRef a = c.sm->args;
-    return ws_ints(c) + ws_regions(c).pads + ((size_t)(layer * 2 + row) * pad_cols(uni(a.hidden_size)) + col) * kPadInts;
+    return uni(c.sm->k.pads) + ((size_t)(layer * 2 + row) * uni(c.sm->k.pad_cols) + col) * kPadInts;
 }
 __device__ __forceinline__ int *shard_ptr(const Ctx &c, int replica, int shard, int layer, int row) {
     const int L = uni(c.sm->args.num_layers);
@@ -804,61 +810,81 @@ __device__ __forceinline__ bool bail(const Ctx &c, int code, int *refusal) {
 // between, and a decode step got 5 % slower.)
 // ---------------------------------------------------------------------------------------------
 struct MatvecDesc {
-    int opcode, layer, ntasks, first_row;
+    int opcode, ntasks, first_row;
     WeightBuffer w0;
     long long gate_delta;  // opcode 5: byte distance from the up matrix (w0) to the gate matrix
     uint32_t row_bytes;
     InsPtr ins;
 };
 
-// false: malformed instruction (nothing has been touched)
-__device__ __forceinline__ bool describe_matvec(SmemPtr sm, int slot, MatvecDesc &d) {
-    ArgsRef a = sm->args;
+// Decodes the matvec instruction in queue slot `slot` (executed once per launch by one thread per
+// slot; the launch arguments come from the kernel's argument registers).
+__device__ __forceinline__ void decode_matvec(SmemPtr sm, int slot, const mk_llama_args &a) {
     const InsPtr ins = sm->queue[slot];
-    const int hid = uni(a.hidden_size), inter = uni(a.intermediate_size);
-    d.ins = ins;
-    d.opcode = uni(ins[0]);
-    d.layer = uni(ins[1]);
+    const int hid = a.hidden_size, inter = a.intermediate_size;
+    const int opcode = ins[0], layer = ins[1];
+    SlotDesc d;
+    d.w0_base = 0;
     d.gate_delta = 0;
-    if (d.layer < 0 || d.layer >= uni(a.num_layers)) return false;
-    if (d.opcode == 1) {
-        const int start = uni(ins[2]), end = uni(ins[3]);
-        const int total_blocks = (uni(a.num_attention_heads) + 2 * uni(a.num_kv_heads)) * uni(a.head_dim) / 16;
-        if (start < 0 || end > total_blocks || end - start > kOutRows / 16) return false;
-        d.ntasks = (end > start ? end - start : 0) * 16;
-        d.first_row = start * 16;
-        d.row_bytes = (uint32_t)hid * 2u;
-        d.w0 = weight_buffer(a.qkv_weights + (size_t)d.layer * total_blocks * 16 * hid, (size_t)total_blocks * 16 * hid * 2);
-        return true;
+    d.w0_bytes = d.row_bytes = 0;
+    d.ntasks = -1;
+    d.first_row = 0;
+    if (layer >= 0 && layer < a.num_layers) {
+        if (opcode == 1) {
+            const int start = ins[2], end = ins[3];
+            const int total_blocks = (a.num_attention_heads + 2 * a.num_kv_heads) * a.head_dim / 16;
+            if (start >= 0 && end <= total_blocks && end - start <= kOutRows / 16) {
+                d.ntasks = (end > start ? end - start : 0) * 16;
+                d.first_row = start * 16;
+                d.row_bytes = (uint32_t)hid * 2u;
+                d.w0_base = (uint64_t)(uintptr_t)(a.qkv_weights + (size_t)layer * total_blocks * 16 * hid);
+                d.w0_bytes = (uint32_t)((size_t)total_blocks * 16 * hid * 2);
+            }
+        } else if (opcode == 4 || opcode == 6) {
+            const bool is_down = opcode == 6;
+            const int start = ins[2], end = ins[3], group = ins[4];
+            const int R = a.matvec_reduction_size, in_dim = is_down ? inter : hid;
+            if (start >= 0 && end <= hid / 16 && group >= 0 && group < in_dim / R && end - start <= kOutRows / 16) {
+                d.ntasks = (end > start ? end - start : 0) * 16;
+                d.first_row = start * 16;
+                d.row_bytes = (uint32_t)in_dim * 2u;
+                // the buffer starts at this column group's first element of the layer's matrix
+                d.w0_base = (uint64_t)(uintptr_t)((is_down ? a.down_weights : a.o_weights) + (size_t)layer * hid * in_dim + (size_t)group * R);
+                d.w0_bytes = (uint32_t)(((size_t)(hid - 1) * in_dim + R) * 2);
+            }
+        } else if (opcode == 5) {
+            const int n = ins[2];
+            bool ok = n >= 0 && n <= MK_INSTRUCTION_WORDS - 3 && n * 32 <= kOutRows;
+            for (int i = 0; ok && i < n; i++) ok = ins[3 + i] >= 0 && ins[3 + i] < inter / 16;
+            if (ok) {
+                d.ntasks = n * 32;
+                d.row_bytes = (uint32_t)hid * 2u;
+                const uint16_t *up = a.up_weights + (size_t)layer * inter * hid;
+                const uint16_t *gate = a.gate_weights + (size_t)layer * inter * hid;
+                d.w0_base = (uint64_t)(uintptr_t)up;
+                d.w0_bytes = (uint32_t)((size_t)inter * hid * 2);
+                d.gate_delta = (long long)((uintptr_t)gate - (uintptr_t)up);
+            }
+        }
     }
-    if (d.opcode == 4 || d.opcode == 6) {
-        const bool is_down = d.opcode == 6;
-        const int start = uni(ins[2]), end = uni(ins[3]), group = uni(ins[4]);
-        const int R = uni(a.matvec_reduction_size), in_dim = is_down ? inter : hid;
-        if (start < 0 || end > hid / 16 || group < 0 || group >= in_dim / R || end - start > kOutRows / 16) return false;
-        d.ntasks = (end > start ? end - start : 0) * 16;
-        d.first_row = start * 16;
-        d.row_bytes = (uint32_t)in_dim * 2u;
-        // the buffer starts at this column group's first element of the layer's matrix
-        d.w0 = weight_buffer((is_down ? a.down_weights : a.o_weights) + (size_t)d.layer * hid * in_dim + (size_t)group * R,
-                             ((size_t)(hid - 1) * in_dim + R) * 2);
-        return true;
-    }
-    if (d.opcode == 5) {
-        const int n = uni(ins[2]);
-        if (n < 0 || n > MK_INSTRUCTION_WORDS - 3 || n * 32 > kOutRows) return false;
-        bool bad = false;
-        for (int i = 0; i < n; i++) bad |= ins[3 + i] < 0 || ins[3 + i] >= inter / 16;
-        if (bad) return false;
-        d.ntasks = n * 32;
-        d.first_row = 0;
-        d.row_bytes = (uint32_t)hid * 2u;
-        d.w0 = weight_buffer(a.up_weights + (size_t)d.layer * inter * hid, (size_t)inter * hid * 2);
-        const uint16_t *gate = uni(a.gate_weights + (size_t)d.layer * inter * hid);
-        d.gate_delta = (long long)((uintptr_t)gate - (uintptr_t)d.w0.base);
-        return true;
-    }
-    return false;
+    MK_LDS u32x4 *dst = (MK_LDS u32x4 *)&sm->desc[slot];
+    dst[0] = u32x4{(uint32_t)d.w0_base, (uint32_t)(d.w0_base >> 32), (uint32_t)d.gate_delta, (uint32_t)((uint64_t)d.gate_delta >> 32)};
+    dst[1] = u32x4{d.w0_bytes, d.row_bytes, (uint32_t)d.ntasks, (uint32_t)d.first_row};
+}
+
+// The decoded form of the matvec instruction in `slot`; false: the instruction is malformed.
+__device__ __forceinline__ bool describe_matvec(SmemPtr sm, int slot, int opcode, MatvecDesc &d) {
+    const MK_LDS u32x4 *src = (const MK_LDS u32x4 *)&sm->desc[slot];
+    const u32x4 lo = src[0], hi = src[1];
+    d.ins = sm->queue[slot];
+    d.opcode = opcode;
+    d.w0.base = (const uint16_t *)(uintptr_t)(((uint64_t)(uint32_t)uni((int)lo.y) << 32) | (uint32_t)uni((int)lo.x));
+    d.gate_delta = (long long)(((uint64_t)(uint32_t)uni((int)lo.w) << 32) | (uint32_t)uni((int)lo.z));
+    d.w0.bytes = (uint32_t)uni((int)hi.x);
+    d.row_bytes = (uint32_t)uni((int)hi.y);
+    d.ntasks = uni((int)hi.z);
+    d.first_row = uni((int)hi.w);
+    return d.ntasks >= 0;
 }
 
 // row computed by task t of the instruction.  Opcode 5: task t is list entry t / 32, matrix
@@ -885,7 +911,7 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
     const int layer = ins[1], start = ins[2], end = ins[3];
     const int hid = a.hidden_size, D = a.head_dim, H = a.num_attention_heads, KVH = a.num_kv_heads;
     const int nblk = end > start ? end - start : 0;
-    const int down_jobs = (a.intermediate_size / a.matvec_reduction_size) * (hid / 16);
+    const int down_jobs = c.sm->k.down_jobs;
     const int k_start = H * D, v_start = k_start + KVH * D;
     constexpr int kPre = 2;
     float rot[kPre][4] = {{1.0f, 1.0f, 0.0f, 0.0f}, {1.0f, 1.0f, 0.0f, 0.0f}};
@@ -1101,7 +1127,7 @@ __device__ __forceinline__ bool control_upgate(const Ctx &c) {
     ArgsRef a = c.sm->args;
     const int layer = ins[1], n = ins[2];
     const int hid = a.hidden_size;
-    const int o_jobs = (hid / a.matvec_reduction_size) * (hid / 16);
+    const int o_jobs = c.sm->k.o_jobs;
     PollTicket ticket = {nullptr, 0, 0};
     uint4 wraw[KC];
     return controller_sequence(
@@ -1133,8 +1159,17 @@ __device__ __forceinline__ bool control_upgate(const Ctx &c) {
                 const float s1 = mkm::round_bf16(mkm::silu_exact(gate[r + 1]));
                 st_u32(a.silu_out + ins[3 + i] * 16 + r, mkm::pack_bf16(s0 * up[r], s1 * up[r + 1]));
             }
+#ifdef MK_TRACE_CONSUMER
+            trace_event(c, 7);
+#endif
             wait_stores();
+#ifdef MK_TRACE_CONSUMER
+            trace_event(c, 8);
+#endif
             signal_sharded(c, layer, 4, n);
+#ifdef MK_TRACE_CONSUMER
+            trace_event(c, 9);
+#endif
         });
 }
 
@@ -1275,7 +1310,7 @@ static __device__ __noinline__ bool op_matvec(SmemPtr lds, int slot, int *refusa
     typedef typename FirstBuffers<PF>::type Map;
     const Ctx c = make_ctx(lds, slot, OP);
     MatvecDesc d;
-    if (!describe_matvec(lds, slot, d)) return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
+    if (!describe_matvec(lds, slot, OP, d)) return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
     if (c.controller) return control_matvec<KC>(c);
     const int mine = rows_of_wave(d.ntasks, c.wave);
     uint4 pool[PF][KC];
@@ -1310,11 +1345,11 @@ static __device__ __noinline__ int op_oproj_upgate(SmemPtr lds, int slot, int *r
     const Ctx co = make_ctx(lds, slot, 4);
     const Ctx cu = make_ctx(lds, slot + 1, 5);
     MatvecDesc dso, dsu;
-    if (!describe_matvec(lds, slot, dso)) {
+    if (!describe_matvec(lds, slot, 4, dso)) {
         bail(co, MK_STATUS_BAD_INSTRUCTION, refusal);
         return 0;
     }
-    const bool pair = describe_matvec(lds, slot + 1, dsu);
+    const bool pair = describe_matvec(lds, slot + 1, 5, dsu);
     if (co.controller) {
         if (!control_matvec<KC>(co)) return 0;
         if (!pair) return 1;
@@ -1337,7 +1372,7 @@ static __device__ __noinline__ int op_oproj_upgate(SmemPtr lds, int slot, int *r
         // and the last row per wave of a down projection that follows directly
         MatvecDesc dsd;
         const bool down_next = MK_PARK_DOWN && KC * 1024 * kConsumerWaves <= kParkBytes && slot + 2 < uni(lds->args.num_slots) &&
-                               uni(lds->queue[slot + 2][0]) == 6 && describe_matvec(lds, slot + 2, dsd);
+                               uni(lds->queue[slot + 2][0]) == 6 && describe_matvec(lds, slot + 2, 6, dsd);
         if (!down_next) dsd = dso;
         const int mine_d = down_next ? rows_of_wave(dsd.ntasks, co.wave) : 0;
         park_rows<KC, 1>(co, (MK_LDS unsigned char *)lds->park + co.wave * (KC * 1024), dsd, mine_d > 0 ? mine_d - 1 : 0, mine_d, down_next);
@@ -1376,7 +1411,7 @@ static __device__ __noinline__ bool op_lm_head(SmemPtr lds, int slot, int *refus
     const int start = ins[1], end = ins[2];
     const int hid = a.hidden_size;
     if (start < 0 || end > a.vocab_size / 16) return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
-    const int down_jobs = (a.intermediate_size / a.matvec_reduction_size) * (hid / 16);
+    const int down_jobs = c.sm->k.down_jobs;
     const int blocks_per_batch = kOutRows / 16;
     const WeightBuffer W = weight_buffer(a.lm_head_weights, (size_t)a.vocab_size * hid * 2);
     float best_v = -INFINITY;
@@ -1426,7 +1461,7 @@ static __device__ __noinline__ bool op_lm_head(SmemPtr lds, int slot, int *refus
         // this worker's maximum logit (the values are bf16-exact) and its first index
         argmax_combine_wave(best_v, best_i);
         if (c.lane == 0 && best_i != INT_MAX) {
-            int *slot_out = ws_ints(c) + ws_regions(c).argmax + 2 * (size_t)c.worker;
+            int *slot_out = uni(c.sm->k.argmax) + 2 * (size_t)c.worker;
             st_i32(slot_out, __builtin_bit_cast(int, best_v));
             st_i32(slot_out + 1, best_i + 1);
         }
@@ -1450,6 +1485,55 @@ __device__ __forceinline__ void halving_level(float *vals, int lane) {
         const uint32_t got = pr.a == own ? pr.b : pr.a;
         vals[k] = keep + __builtin_bit_cast(float, got);
     }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Log-sum-exp merge of n attention partitions of one head (python_vm.py:349-393), executed by the
+// D/2 threads of the head (thread j: output dims 2j and 2j + 1, and the log-sum-exp of list entry
+// j).  All 64 lanes of the wave must be active; with D = 64 the wave holds two heads.  `list_at(k)`
+// is the partition index of list entry k.  Returns the merged pair and log-sum-exp; the caller stores.
+// ---------------------------------------------------------------------------------------------
+struct MergedPair {
+    float o0, o1, lse;
+};
+template <int D, class ListAt>
+__device__ __forceinline__ MergedPair merge_partitions(const Ctx &c, int head, int j, int n_any, ListAt list_at) {
+    constexpr int kMaxList = MK_INSTRUCTION_WORDS - 7;
+    constexpr int TPH = D / 2;
+    ArgsRef a = c.sm->args;
+    const int n = uni(n_any);  // the same for the whole wave: the loops below branch on scalars
+    const int MP = uni(a.max_partials), d = j * 2;
+    const float *outs = a.attn_out_intermediates + (size_t)head * MP * D + d;
+    const float *lses = a.attn_lse_intermediates + (size_t)head * MP;
+    // lane j of a head's lane group holds list entry j: its partition index and log-sum-exp
+    const int entry = j < n ? list_at(j) : 0;
+    const float lse = j < n ? ld_f32(lses + entry) : -INFINITY;
+    // every request goes out at once: this thread's two dims of each listed partition
+    uint64_t v[kMaxList];
+#pragma unroll
+    for (int k = 0; k < kMaxList; k++)
+        if (k < n) v[k] = ld_u64(outs + (size_t)__builtin_amdgcn_readlane(entry, k) * D);
+    // weights 2^(lse_i - max)
+    const float m = lane_tree_max<1, TPH>(lse);
+    const float wj = j < n ? mkm::exp2f_exact(lse - m) : 0.0f;
+    float den = 0.0f, o0 = 0.0f, o1 = 0.0f;
+    // accumulate in list order; entry k's weight comes from lane k of this head's group
+#pragma unroll
+    for (int k = 0; k < kMaxList; k++)
+        if (k < n) {
+            float w;
+            if constexpr (TPH == 64) {
+                w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), k));
+            } else {
+                const float w_lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), k));
+                const float w_hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), k + 32));
+                w = c.lane < 32 ? w_lo : w_hi;
+            }
+            den = den + w;
+            o0 = fmaf(w, mkm::bits_f32((uint32_t)v[k]), o0);
+            o1 = fmaf(w, mkm::bits_f32((uint32_t)(v[k] >> 32)), o1);
+        }
+    return MergedPair{o0 / den, o1 / den, m + mkm::log2f_exact(den)};
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1497,6 +1581,7 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
                                       false, D / 16);
         trace_event(c, kEvDepReady);
         if (!barrier_inputs_ready(c, ok)) return false;
+        trace_event(c, kEvInputReady);
         wg_barrier();  // wave maxima
         trace_event(c, 6);
         wg_barrier();  // probabilities
@@ -1744,81 +1829,55 @@ static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot
     const InsPtr ins = lds->queue[slot];
     const Ctx c = make_ctx(lds, slot, ins[0]);
     ArgsRef a = c.sm->args;
-    const SmemPtr sm = c.sm;
     constexpr int kMaxList = MK_INSTRUCTION_WORDS - 7;
     constexpr int TPH = D / 2;  // threads per head, two output dims each; all in one wave
     static_assert(TPH >= kMaxList && TPH <= 64, "a head's threads also fetch one list entry's log-sum-exp each");
-    const int layer = ins[1], hs = ins[2], P = ins[3], terminal = ins[4], n = ins[5];
-    const int R = a.attn_reduction_size, MP = a.max_partials;
+    const int layer = uni(ins[1]), hs = uni(ins[2]), P = uni(ins[3]), terminal = uni(ins[4]), n = uni(ins[5]);
+    const int R = uni(a.attn_reduction_size), MP = uni(a.max_partials);
     bool bad = layer < 0 || layer >= a.num_layers || n < 1 || n > kMaxList || hs < 0 ||
                hs + R > a.num_attention_heads || R > kGqa || a.head_dim != D;
-    if (!bad)
-        for (int i = 0; i < n; i++) bad |= ins[6 + i] < 0 || ins[6 + i] >= MP;
-    const int out_idx = bad ? 0 : ins[6 + n];
+    // the listed partitions, one per lane
+    if (!bad) bad = __any(c.lane < n && (ins[6 + c.lane] < 0 || ins[6 + c.lane] >= MP)) != 0;
+    const int out_idx = bad ? 0 : uni(ins[6 + n]);
     bad |= !terminal && (out_idx < 0 || out_idx >= MP);
     if (bad) return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
 
-    if (c.controller) {
-        const bool mine = c.lane < R;
-        const bool ok = poll_counters(c, mine ? pad_ptr(c, layer, 1, hs + c.lane) : nullptr,
-                                      mine ? bar_ptr(c, layer, 1, hs + c.lane) : nullptr, false, P);
-        trace_event(c, kEvDepReady);
-        if (!barrier_inputs_ready(c, ok)) return false;
-        trace_event(c, kEvComputeDone);
-        // the waves that merge the partitions store and signal on their own
-        return true;
-    }
-    if (!barrier_inputs_ready(c, true)) return false;
+    // The waves that hold the heads' threads wait for their own heads' partitions, merge, store and
+    // signal; nobody else has anything to do.  (No weights are streamed here, so a wave's looks at
+    // the counters do not queue behind bulk loads of its own.)  Everybody leaves together, after the
+    // signal: the next instruction starts with bulk weight requests, and a CU serves its requests in
+    // order.
     if (c.tid < R * TPH) {
         const int h = c.tid / TPH, j = c.tid % TPH, d = j * 2;
         const int head = hs + h;
-        const float *outs = a.attn_out_intermediates + (size_t)head * MP * D;
-        const float *lses = a.attn_lse_intermediates + (size_t)head * MP;
-        // every request goes out at once: this thread's two dims of each listed partition, and the
-        // log-sum-exp of list entry j
-        const float lse = j < n ? ld_f32(lses + ins[6 + j]) : -INFINITY;
-        uint64_t v[kMaxList];
-#pragma unroll
-        for (int k = 0; k < kMaxList; k++)
-            if (k < n) v[k] = ld_u64(outs + (size_t)ins[6 + k] * D + d);
-        // weights 2^(lse_i - max): lane j of the head's lane group holds the weight of list entry j
-        const float m = lane_tree_max<1, TPH>(lse);
-        const float wj = j < n ? mkm::exp2f_exact(lse - m) : 0.0f;
-        trace_consumer(c, 26);
-        float den = 0.0f, o0 = 0.0f, o1 = 0.0f;
-        // accumulate in list order; entry k's weight comes from lane k of this head's group
-#pragma unroll
-        for (int k = 0; k < kMaxList; k++)
-            if (k < n) {
-                float w;
-                if constexpr (TPH == 64) {
-                    w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), k));
-                } else {
-                    const float w_lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), k));
-                    const float w_hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), k + 32));
-                    w = c.lane < 32 ? w_lo : w_hi;
-                }
-                den = den + w;
-                o0 = fmaf(w, mkm::bits_f32((uint32_t)v[k]), o0);
-                o1 = fmaf(w, mkm::bits_f32((uint32_t)(v[k] >> 32)), o1);
+        const bool leader = j == 0;
+        const PollTicket ticket =
+            poll_issue(c, leader ? pad_ptr(c, layer, 1, head) : nullptr, leader ? bar_ptr(c, layer, 1, head) : nullptr);
+        if (poll_wait(c, ticket, false, P, []() {})) {
+            trace_consumer(c, 26);
+            const MergedPair r = merge_partitions<D>(c, head, j, n, [&](int k) { return ins[6 + k]; });
+            trace_consumer(c, 27);
+            if (terminal) {
+                st_u32(a.attn_out + (size_t)head * D + d, mkm::pack_bf16(r.o0, r.o1));
+            } else {
+                float *dst = a.attn_out_intermediates + ((size_t)head * MP + out_idx) * D + d;
+                st_f32(dst, r.o0);
+                st_f32(dst + 1, r.o1);
+                if (leader) st_f32(a.attn_lse_intermediates + (size_t)head * MP + out_idx, r.lse);
             }
-        trace_consumer(c, 27);
-        o0 = o0 / den;
-        o1 = o1 / den;
-        if (terminal) {
-            st_u32(a.attn_out + (size_t)head * D + d, mkm::pack_bf16(o0, o1));
-        } else {
-            float *dst = a.attn_out_intermediates + ((size_t)head * MP + out_idx) * D + d;
-            st_f32(dst, o0);
-            st_f32(dst + 1, o1);
-            if (j == 0) st_f32(a.attn_lse_intermediates + (size_t)head * MP + out_idx, m + mkm::log2f_exact(den));
+            wait_stores();
+            if (leader) signal_sharded_lane(c, layer, 2, 1);
+            trace_consumer(c, 28);
+            trace_consumer_flush(c, 26, 28);
+        } else if (c.lane == 0) {
+            c.sm->abort = 1;
         }
-        wait_stores();
-        trace_consumer(c, 28);
-        if (j == 0) signal_sharded_lane(c, layer, 2, 1);
-        trace_consumer_flush(c, 26, 28);
     }
-    return true;
+    wg_barrier();
+    trace_event(c, kEvDepReady);
+    trace_event(c, kEvInputReady);
+    trace_event(c, kEvComputeDone);
+    return c.sm->abort == 0;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1833,7 +1892,6 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
         sm->abort = 0;
         sm->last_flag = 0;
         sm->parked_slot = -1;
-        sm->t_launch = wall_clock64();
         // the token whose embedding row starts the step (written by the previous launch or the host)
         int token = -1;
         if (a.token_in) {
@@ -1858,6 +1916,30 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
         const int words = a.num_slots * MK_INSTRUCTION_WORDS;
         MK_LDS int *dst = &sm->queue[0][0];
         for (int i = tid; i < words; i += kThreads) dst[i] = queue[i];
+    }
+    if (tid == 0) {
+        int *const ws = static_cast<int *>(a.workspace);
+        const WsLayout w = ws_layout(a.num_layers, a.hidden_size, a.intermediate_size, a.matvec_reduction_size);
+        sm->k.status = ws + w.status;
+        sm->k.shards = ws + w.shards;
+        sm->k.arrive_o = ws + w.arrive_o;
+        sm->k.arrive_d = ws + w.arrive_d;
+        sm->k.argmax = ws + w.argmax;
+        sm->k.pads = ws + w.pads;
+        sm->k.partial = reinterpret_cast<float *>(ws + w.partial);
+        sm->k.trace_base =
+            (a.flags & MK_FLAG_TIMINGS) && a.timings ? a.timings + (size_t)blockIdx.x * a.num_slots * MK_TIMING_SLOTS : nullptr;
+        sm->k.spin_ticks = (long long)(a.spin_limit_us ? a.spin_limit_us : 2000000u) * 100;  // 100 MHz wall clock
+        sm->k.cols = a.num_attention_heads + 2 * a.num_kv_heads;
+        sm->k.pad_cols = pad_cols(a.hidden_size);
+        sm->k.down_jobs = (a.intermediate_size / a.matvec_reduction_size) * (a.hidden_size / 16);
+        sm->k.o_jobs = (a.hidden_size / a.matvec_reduction_size) * (a.hidden_size / 16);
+    }
+    wg_barrier();
+    // decode the matvec instructions of the queue, one thread per slot
+    for (int slot = tid; slot < a.num_slots; slot += kThreads) {
+        const int opcode = sm->queue[slot][0];
+        if (opcode == 1 || (opcode >= 4 && opcode <= 6)) decode_matvec(sm, slot, a);
     }
     wg_barrier();
 

@@ -388,3 +388,42 @@ class LatencyScheduleBuilder(ScheduleBuilder):
             schedule,
             globs=cls.make_globals(model, skip_attn_reduction=schedule.globs.skip_attn_reduction),
         )
+
+
+def compute_unit_assign_to_sms(instructions: list[Instruction], sm_count: int):
+    """Assignment policy ``"cu"`` (no counterpart in the reference, whose policies are in
+    ``scheduler.py:94-271``): round robin within each run of equal opcodes, except that a layer's
+    short, latency-bound chain - attention partitions, partition merges, O projections - is spread
+    so that the O-projection blocks avoid the workers that have just run a full attention partition.
+
+    Attention partitions go to the first workers, merges to the next ones, and every O-projection
+    block to the worker that has the least of the chain so far: first the idle workers, then the
+    merge workers, then workers whose partition was the last of its head (the remainder of the
+    division into partitions, often a handful of tokens), then the others; nobody gets a second
+    block before everybody has one.  With 256 workers and 17 partitions the 128 blocks land on the
+    112 idle workers, the 8 merge workers and the 8 workers with a remainder partition.  Under round
+    robin 16 of them fall to workers that have just run a full partition; those see the O
+    projection's dependency late, behind their own weight requests, and every worker then waits for
+    them.  The linear order of the instructions, and with it every barrier count, is unchanged."""
+    from megakernels_amd.scheduler import collect_into_waves
+
+    queues: list[list[Instruction]] = [[] for _ in range(sm_count)]
+    chain_load = [0] * sm_count
+    O_PROJ, MERGE, ATTENTION, REMAINDER = 1_000_000, 1_100, 1_000, 900
+    for wave in collect_into_waves(instructions):
+        opcode = wave[0].opcode()
+        if opcode == PartialAttention.opcode():
+            chain_load = [0] * sm_count   # a new layer's chain starts
+        if opcode in (PartialAttention.opcode(), AttentionReduction.opcode(), O_ProjResidual.opcode()):
+            for ins in wave:
+                if opcode == PartialAttention.opcode():
+                    weight = REMAINDER if ins.partial_idx == ins.num_partials - 1 and ins.num_partials > 1 else ATTENTION
+                else:
+                    weight = MERGE if opcode == AttentionReduction.opcode() else O_PROJ
+                worker = min(range(sm_count), key=lambda w: (chain_load[w], w))
+                chain_load[worker] += weight
+                queues[worker].append(ins)
+        else:
+            for i, ins in enumerate(wave):
+                queues[i % sm_count].append(ins)
+    return queues

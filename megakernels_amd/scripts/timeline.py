@@ -13,7 +13,8 @@ reference's ``diff_test.py outfile=`` dump (``scripts/diff_test.py:231-242``).  
 same events (``include/util.cuh:215-246``) when compiled with ``TIMING_RECORD_ENABLED``; here the records
 are taken on request at run time.
 
-Times are microseconds since the workgroup started (100 MHz wall clock of the device).
+Times are microseconds since the first workgroup took its first instruction (100 MHz wall clock of the
+device, common to all compute units).
 """
 
 from __future__ import annotations
@@ -83,7 +84,10 @@ def main(argv):
     # [workers, slots, 6]: start, dependency seen, activation ready, rows done, end, opcode
     t = globs.timings.cpu()[:, :, :6].numpy().astype(np.float64)
     ins = globs.instructions.cpu().numpy()
-    t[:, :, :5] /= 100.0
+    # the records are the low 32 bits of the device clock: times since the earliest record
+    executed = t[:, :, 5] != 0
+    origin = np.int64(globs.timings.cpu()[:, :, 0].numpy()[executed].astype(np.uint32).min())
+    t[:, :, :5] = ((t[:, :, :5].astype(np.int64) - origin) % (1 << 32)) / 100.0
     if opts["out"]:
         np.savez_compressed(opts["out"], timings=globs.timings.cpu().numpy(), instructions=ins,
                             ticks_per_microsecond=np.array(100))

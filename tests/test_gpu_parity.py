@@ -127,6 +127,12 @@ def test_tiny_split_kv_layer_started_after_the_reduction():
     _suffix_case(config_tiny(), workers=16, pos=44, start_after_op="reduction", partitions=3)
 
 
+def test_tiny_split_kv_layer_started_after_the_partitions():
+    # the partitions were counted in `barriers` before the launch: the reduction instructions do the
+    # merging themselves although the schedule would let the last partition do it
+    _suffix_case(config_tiny(), workers=16, pos=44, start_after_op="partial", partitions=3)
+
+
 def test_1b_slice_layer_started_after_the_o_projection():
     _suffix_case(config_1b_slice(layers=2), workers=256, pos=70, start_after_op="oproj")
 
