@@ -12,11 +12,15 @@ reference's sequence of small kernels around a launch per token instead.
 Weights, KV cache and instruction tensor are resident in HBM before the timed
 region starts.
 
-Workloads (all Llama-3.2-1B architecture, random bf16 weights N(0, 0.02) from
-seed 0, RMSNorm weights 1):
-  c1  32-token prompt prefilled by the plain PyTorch forward, decode from position 32
-  c2  KV cache pre-filled to 4096 positions with seeded N(0,1), decode from position 4096  (default)
-  c3  KV cache pre-filled to 16384 positions
+Workloads (random bf16 weights N(0, 0.02) from seed 0, RMSNorm weights 1):
+  c1  Llama-3.2-1B architecture, 32-token prompt prefilled by the plain PyTorch forward, decode from position 32
+  c2  1B, KV cache pre-filled to 4096 positions with seeded N(0,1), decode from position 4096  (default)
+  c3  1B, KV cache pre-filled to 16384 positions
+  c4  Llama-3.1-8B architecture (untied LM head), 32-token prompt, decode from position 32
+  c5  8B, KV cache pre-filled to 32768 positions
+The 1B weights come from the CPU generator; the 8B weights (7.5 G parameters) and the long KV
+pre-fills are drawn by the GPU's generator, which takes seconds instead of minutes.  The prompt
+prefill runs on the GPU, outside the timed region, and its cache is what the CPU checker starts from.
 
 Prints one JSON line.  `roofline` prices the megakernel alone: algorithmic
 bytes per launch (weights + norm weights + K/V read, summed over the steps of
@@ -41,6 +45,15 @@ sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBPS = 8000.0
 
+# prefill: cached positions when decoding starts; kv: where they come from
+WORKLOADS = {
+    "c1": {"arch": "1b", "prefill": 32, "kv": "prompt"},
+    "c2": {"arch": "1b", "prefill": 4096, "kv": "random"},
+    "c3": {"arch": "1b", "prefill": 16384, "kv": "random"},
+    "c4": {"arch": "8b", "prefill": 32, "kv": "prompt"},
+    "c5": {"arch": "8b", "prefill": 32768, "kv": "random"},
+}
+
 
 def algorithmic_bytes(cfg, pos: int) -> int:
     """Bytes one decode step must read at least: bf16 matrices (tied embedding
@@ -60,8 +73,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3"])
-    ap.add_argument("--cpu-steps", type=int, default=32, help="decode steps timed on the CPU checker (0 = skip)")
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-steps", type=int, default=-1,
+                    help="decode steps timed on the CPU checker (0 = skip; default 32 for the 1B workloads, 4 for 8B)")
+    ap.add_argument("--torch-steps", type=int, default=-1,
+                    help="decode steps also timed on the torch restatement of the Python VM, the closer stand-in for "
+                         "the reference's python_vm.py (0 = skip; default 3 for 1B, 1 for 8B)")
     ap.add_argument("--sched", default="rr")
     ap.add_argument("--partitions", type=int, default=0, help="attention partitions (0 = one per 256 positions, max 24)")
     ap.add_argument("--loop", default="fused", choices=["fused", "reference"],
@@ -98,33 +115,45 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
-    cfg = LlamaConfig.llama_1b()
+    work = WORKLOADS[args.workload]
+    big = work["arch"] == "8b"
+    cfg = LlamaConfig.llama_8b() if big else LlamaConfig.llama_1b()
     total_steps = args.warmup + args.steps
-    prefill = {"c1": 32, "c2": 4096, "c3": 16384}[args.workload]
+    prefill = work["prefill"]
     max_len = prefill + total_steps + 16
+    cpu_steps = args.cpu_steps if args.cpu_steps >= 0 else (4 if big else 32)
+    torch_steps = args.torch_steps if args.torch_steps >= 0 else (1 if big else 3)
+    need_cpu_twin = cpu_steps > 0 or torch_steps > 0
     t_setup = time.time()
-    model_cpu = LlamaForCausalLM.from_random(cfg, ExtraModelConfig(interleave_rope=True, max_len_override=max_len), seed=0)
+    extra = ExtraModelConfig(interleave_rope=True, max_len_override=max_len)
+    if big:
+        model = LlamaForCausalLM.from_random(cfg, extra, seed=0, device=device, draw_device=device)
+        model_cpu = model.to("cpu") if need_cpu_twin else None
+    else:
+        model_cpu = LlamaForCausalLM.from_random(cfg, extra, seed=0)
+        model = model_cpu.to(device)
 
     prompt_gen = torch.Generator().manual_seed(1)
     prompt = torch.randint(0, cfg.vocab_size, (1, 32), generator=prompt_gen)
-    if args.workload == "c1":
-        # prefill once with the plain forward; both the GPU and the checker start from its cache
-        out = model_cpu(BatchState(input_ids=prompt, position_ids=torch.arange(32)))
+    if work["kv"] == "prompt":
+        # prefill once with the plain forward on the GPU (reference scripts/generate.py:125-137); the
+        # megakernel and the checker both start from its cache
+        out = model(BatchState(input_ids=prompt.to(device), position_ids=torch.arange(32, device=device)))
         first_token = int(out.output_ids[0, -1])
     else:
-        kv_gen = torch.Generator().manual_seed(2)
-        for cache in model_cpu.stacked_kv_cache:
-            shape = list(cache.shape)
-            shape[2] = prefill
-            cache[:, :, :prefill] = torch.randn(shape, generator=kv_gen).to(cache.dtype)
+        kv_gen = torch.Generator(device=device).manual_seed(2)
+        for cache in model.stacked_kv_cache:
+            for layer in range(cache.shape[0]):
+                rows = torch.randn((cache.shape[1], prefill) + tuple(cache.shape[3:]), generator=kv_gen, device=device)
+                cache[layer, :, :prefill] = rows.to(cache.dtype)
         first_token = int(prompt[0, 0])
+    if model_cpu is not None:
+        for dst, src in zip(model_cpu.stacked_kv_cache, model.stacked_kv_cache):
+            dst.copy_(src)
 
     workers = get_sm_count(device)
     set_sm_count_override(workers)
     partitions = args.partitions or pick_num_attention_partitions(prefill, total_steps)
-    model = model_cpu.to(device)
-    for dst, src in zip(model.stacked_kv_cache, model_cpu.stacked_kv_cache):
-        dst.copy_(src)
 
     schedule = LatencyScheduleBuilder.build(model, num_attention_partitions=partitions)
     tensorize_instructions(schedule.globs, assign_to_sms(args.sched, schedule=schedule))
@@ -204,10 +233,10 @@ def main():
     # ---- CPU baseline: the checker on the same decode steps (bounded sample) --
     cpu_baseline = None
     parity = None
-    if args.cpu_steps > 0:
+    if cpu_steps > 0:
         from oracle import pyvm
 
-        n_cpu = min(args.cpu_steps, total_steps)
+        n_cpu = min(cpu_steps, total_steps)
         set_sm_count_override(workers)
         schedule_cpu = LatencyScheduleBuilder.build(model_cpu, num_attention_partitions=partitions)
         oracle_gen = pyvm.OracleGenerator(model_cpu, schedule_cpu)
@@ -229,18 +258,48 @@ def main():
         got = tokens_gpu[: n_cpu + 1]
         agree = sum(int(a == b) for a, b in zip(expect, got))
         parity = {"tokens_compared": n_cpu + 1, "tokens_equal": agree, "bit_exact": agree == n_cpu + 1}
+        if torch_steps > 0:
+            # the same steps once more on the restatement written with the reference's own torch calls
+            # (one small bf16 matvec per 16-row block, as megakernels/demos/latency/python_vm.py does):
+            # what the reference's Python VM costs on these cores
+            from oracle import pyvm_torch
+
+            n_torch = min(torch_steps, n_cpu)
+            globs = schedule_cpu.globs
+            instructions = schedule_cpu.get_linear_instructions()
+            embed = model_cpu.model.embed_tokens.weight
+            for dst, src in zip(model_cpu.stacked_kv_cache, model.stacked_kv_cache):
+                dst.copy_(src)   # the checker appended rows; start from the same cache again
+            tt0 = time.perf_counter()
+            for i in range(n_torch):
+                globs.hidden_states[:] = embed[int(tokens_cpu[0, i])]
+                globs.barriers.zero_()
+                globs.pos_id = prefill + i
+                pyvm_torch.interpret(globs, instructions)
+            torch_elapsed = time.perf_counter() - tt0
+            cpu_baseline["torch_restatement"] = {
+                "value": round(n_torch / torch_elapsed, 4),
+                "unit": "tokens/s",
+                "cores": torch.get_num_threads(),
+                "kind": "torch-restatement",
+                "sample": f"first {n_torch} decode step(s), torch.set_num_threads default ({torch.get_num_threads()}), "
+                          f"{torch_elapsed:.1f} s",
+                "us_per_step": round(torch_elapsed / n_torch * 1e6, 1),
+            }
 
     # HBM bytes per launch measured with rocprofv3 --pmc for this workload (committed summary)
     traffic = None
+    traffic_source = None
     traffic_file = ROOT / "profiles" / f"mk_llama_kernel_{args.workload}_traffic.json"
     if traffic_file.exists():
+        traffic_source = f"committed rocprofv3 --pmc summary profiles/{traffic_file.name} (not measured in this run)"
         measured = json.loads(traffic_file.read_text())
         # the counters were taken per launch of `steps_per_launch` steps
         per_step = (measured["fetch_bytes_per_launch"] + measured["write_bytes_per_launch"]) / measured.get("steps_per_launch", 1)
         traffic = int(per_step * usual)
 
     result = {
-        "metric": "batch-1 decode tokens/s (Llama-3.2-1B arch)",
+        "metric": f"batch-1 decode tokens/s ({'Llama-3.1-8B' if big else 'Llama-3.2-1B'} arch)",
         "value": round(args.steps / elapsed, 2),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -253,9 +312,11 @@ def main():
         "dtype": "bf16",
         "data": "synthetic",
         "config": {
-            "workload": f"{args.workload}: Llama-3.2-1B architecture, random-init bf16 weights (seed 0), batch 1, "
-                        f"KV pre-filled to {prefill} positions, greedy decode of {args.steps} timed tokens "
-                        f"from position {first_pos}",
+            "workload": f"{args.workload}: {'Llama-3.1-8B' if big else 'Llama-3.2-1B'} architecture, random-init bf16 "
+                        f"weights (seed 0, {'GPU' if big else 'CPU'} generator), batch 1, "
+                        + (f"32-token prompt prefilled on the GPU, " if work["kv"] == "prompt" else
+                           f"KV pre-filled to {prefill} positions with seeded N(0,1), ")
+                        + f"greedy decode of {args.steps} timed tokens from position {first_pos}",
             "workers": workers,
             "attention_partitions": partitions,
             "assignment": args.sched,
@@ -270,7 +331,8 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved_gbps / HBM_PEAK_GBPS, 4),
             "traffic": traffic,
-            "kernel": "mk_llama_kernel<4,4,64>",
+            "traffic_source": traffic_source,
+            "kernel": "mk_llama_kernel<8,4,128>" if big else "mk_llama_kernel<4,4,64>",
             "kernel_us": round(kernel_ms_mean * 1e3, 2),
             "kernel_us_per_step": round(kernel_ms_mean * 1e3 / usual, 2),
             "launches_timed": len(usual_ms),

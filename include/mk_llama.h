@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define MK_LLAMA_ABI_VERSION 4
+#define MK_LLAMA_ABI_VERSION 5
 #define MK_INSTRUCTION_WORDS 32   /* megakernels/scheduler.py:13, include/config.cuh:14 */
 #define MK_TIMING_SLOTS 128       /* megakernels/scheduler.py:14, include/config.cuh:18 */
 #define MK_BARRIER_ROWS 10        /* megakernels/demos/latency/scheduler.py:53-61 */
@@ -62,7 +62,7 @@ enum {
     MK_STATUS_OK = 0,
     MK_STATUS_BARRIER_TIMEOUT = 1,   /* a barrier wait exceeded spin_limit_us */
     MK_STATUS_BAD_OPCODE = 2,        /* reference: asm trap, include/util.cuh:38 */
-    MK_STATUS_ATTN_TOO_LONG = 3,     /* one attention partition exceeds the on-chip score buffer */
+    MK_STATUS_ATTN_TOO_LONG = 3,     /* reserved: partitions of any length run since ABI version 5 */
     MK_STATUS_BAD_INSTRUCTION = 4,   /* field out of range for the given shapes */
     MK_STATUS_BAD_TOKEN = 5          /* *token_in outside the vocabulary */
 };
@@ -161,7 +161,8 @@ int mk_llama_read_status(void *workspace, void *hip_stream, int32_t out[4]);
 
 /* what = 0: compute units of the current device; 1: LDS bytes the kernel
  * requests per workgroup; 2: threads per workgroup; 3: ABI version; 4: longest
- * attention partition (tokens) the kernel accepts. */
+ * attention partition (tokens) whose scores stay on the chip - a longer one is
+ * accepted and recomputes its scores in the second pass. */
 int mk_llama_query(int what);
 
 /* Self test (no counterpart in the reference): counts the binary32 inputs, over all 2^32 bit

@@ -69,7 +69,7 @@ constexpr int kHotRows = 4;         // barrier rows 2..5 are sharded
 constexpr int kOutRows = 2048;      // rows staged in LDS between matvec and epilogue
 constexpr int kMaxK = 4096;         // longest activation vector handed through LDS
 constexpr int kScoreCap = 4096;     // tokens per attention partition (LDS score buffer)
-constexpr int kQueueSlots = 192;    // longest instruction queue per worker (kept in LDS)
+constexpr int kQueueSlots = 192;    // instructions of a worker's queue kept in LDS at a time (a longer queue goes through in windows)
 constexpr int kParkBytes = kConsumerWaves * 4096;  // one more parked row per wave, outside the score buffer
 constexpr int kMaxHeadDim = 128;
 constexpr int kGqa = 4;             // query heads per KV head handled by one attention instruction
@@ -99,8 +99,11 @@ constexpr int kStepSlot = 9;        // workspace int: decode steps of this launc
 #ifndef MK_PF_LMHEAD
 #define MK_PF_LMHEAD 2
 #endif
+#ifndef MK_PF_WIDE_CAP
+#define MK_PF_WIDE_CAP 2
+#endif
 template <int KC>
-constexpr int rows_in_flight(int wanted) { return KC <= 4 ? wanted : (wanted < 2 ? wanted : 2); }
+constexpr int rows_in_flight(int wanted) { return KC <= 4 ? wanted : (wanted < MK_PF_WIDE_CAP ? wanted : MK_PF_WIDE_CAP); }
 
 #ifndef MK_PAIR_OPROJ_UPGATE
 #define MK_PAIR_OPROJ_UPGATE 1      // O-proj and a directly following up/gate run as one handler
@@ -175,6 +178,7 @@ struct Smem {
     int abort;                      // set once, never cleared during a launch
     int last_flag;
     int token;                      // *token_in, or -1
+    int window_base, window_count;  // which slots of the worker's queue are in `queue` / `desc`: [base, base + count)
     Consts k;
     mk_llama_args args;             // the launch arguments, read from here by every instruction
     int flags[kOutRows / 16];       // per-block "I was the last arriver" (matvec-add)
@@ -189,8 +193,8 @@ struct Smem {
     alignas(16) float scores[kScoreCap][kGqa];  // attention: one partition's scores, then probabilities
     alignas(16) unsigned char park[kParkBytes];  // a weight row per wave parked for a later instruction
     int parked_slot;                               // the instruction whose last row per wave lies in `park`, or -1
-    alignas(16) SlotDesc desc[kQueueSlots];        // the matvec instructions of the queue, decoded once
-    alignas(16) int queue[kQueueSlots][MK_INSTRUCTION_WORDS];  // this worker's instructions, fetched once
+    alignas(16) SlotDesc desc[kQueueSlots];        // the matvec instructions of the window, decoded
+    alignas(16) int queue[kQueueSlots][MK_INSTRUCTION_WORDS];  // a window of this worker's instructions
 };
 static_assert(offsetof(Smem, x) % 16 == 0 && offsetof(Smem, wave_max) % 16 == 0 && offsetof(Smem, wave_l) % 16 == 0 &&
                   offsetof(Smem, scores) % 16 == 0,
@@ -406,7 +410,7 @@ struct Ctx {
     SmemPtr sm;
     int tid, wave, lane;
     bool controller;
-    int worker, slot, opcode;
+    int worker, slot, opcode;       // slot: index into the window of the queue that is in LDS
     int *trace;                     // this instruction's timing row, or nullptr when tracing is off
 };
 
@@ -421,7 +425,7 @@ __device__ __forceinline__ Ctx make_ctx(SmemPtr sm, int slot, int opcode) {
     c.slot = slot;
     c.opcode = opcode;
     int *const rows = uni(sm->k.trace_base);
-    c.trace = rows ? rows + (size_t)slot * MK_TIMING_SLOTS : nullptr;
+    c.trace = rows ? rows + (size_t)(uni(sm->window_base) + slot) * MK_TIMING_SLOTS : nullptr;
     return c;
 }
 
@@ -482,7 +486,7 @@ __device__ void record_status(const Ctx &c, int code) {
     int *status = ws_status(c);
     if (__hip_atomic_compare_exchange_strong(as_global(&status[0]), &expected, code, __ATOMIC_RELAXED, __ATOMIC_RELAXED, AG)) {
         st_i32(&status[1], c.worker);
-        st_i32(&status[2], c.slot);
+        st_i32(&status[2], c.sm->window_base + c.slot);
         st_i32(&status[3], c.opcode);
     }
 }
@@ -1159,17 +1163,8 @@ __device__ __forceinline__ bool control_upgate(const Ctx &c) {
                 const float s1 = mkm::round_bf16(mkm::silu_exact(gate[r + 1]));
                 st_u32(a.silu_out + ins[3 + i] * 16 + r, mkm::pack_bf16(s0 * up[r], s1 * up[r + 1]));
             }
-#ifdef MK_TRACE_CONSUMER
-            trace_event(c, 7);
-#endif
             wait_stores();
-#ifdef MK_TRACE_CONSUMER
-            trace_event(c, 8);
-#endif
             signal_sharded(c, layer, 4, n);
-#ifdef MK_TRACE_CONSUMER
-            trace_event(c, 9);
-#endif
         });
 }
 
@@ -1371,7 +1366,7 @@ static __device__ __noinline__ int op_oproj_upgate(SmemPtr lds, int slot, int *r
         park_rows<KC, kParked>(co, slice, dsu, mine_u > kParked ? mine_u - kParked : 0, mine_u, pair);
         // and the last row per wave of a down projection that follows directly
         MatvecDesc dsd;
-        const bool down_next = MK_PARK_DOWN && KC * 1024 * kConsumerWaves <= kParkBytes && slot + 2 < uni(lds->args.num_slots) &&
+        const bool down_next = MK_PARK_DOWN && KC * 1024 * kConsumerWaves <= kParkBytes && slot + 2 < uni(lds->window_count) &&
                                uni(lds->queue[slot + 2][0]) == 6 && describe_matvec(lds, slot + 2, 6, dsd);
         if (!down_next) dsd = dso;
         const int mine_d = down_next ? rows_of_wave(dsd.ntasks, co.wave) : 0;
@@ -1533,6 +1528,9 @@ __device__ __forceinline__ MergedPair merge_partitions(const Ctx &c, int head, i
             o0 = fmaf(w, mkm::bits_f32((uint32_t)v[k]), o0);
             o1 = fmaf(w, mkm::bits_f32((uint32_t)(v[k] >> 32)), o1);
         }
+    // every listed partition empty (a run past the end of the sequence in a reduction tree): the merge
+    // of nothing is nothing, as for an empty partition itself
+    if (m == -INFINITY) return MergedPair{0.0f, 0.0f, -INFINITY};
     return MergedPair{o0 / den, o1 / den, m + mkm::log2f_exact(den)};
 }
 
@@ -1569,7 +1567,8 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
     const int t0 = sb * 16;
     const int t1 = min(eb * 16, seq_len);
     const int T = t1 > t0 ? t1 - t0 : 0;
-    if (T > kScoreCap) return bail(c, MK_STATUS_ATTN_TOO_LONG, refusal);
+    // a partition longer than the score buffer works without it: its second pass recomputes the scores
+    const bool scores_fit = T <= kScoreCap;
     const int h0 = kvh * G;
     const int rounds = (T + NSLOT - 1) / NSLOT;
 
@@ -1645,34 +1644,49 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
     }
     trace_consumer(c, 17);
 
-    // ---- pass 1: scores (kept as [token][head] in LDS) and maximum ----
+    // scores of one token against the four heads, valid in all lanes of the token's group
+    auto scores_of = [&](const uint4 &krow, float (&sc)[G]) {
+        float kf[8];
+        unpack8(krow, kf);
+#pragma unroll
+        for (int h = 0; h < G; h++) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc = fmaf(q[h][e], kf[e], acc);
+            sc[h] = group_tree_sum<LPT>(acc) * a.attn_scale;
+        }
+    };
+
+    // ---- pass 1: scores (kept as [token][head] in LDS when the partition fits) and maximum ----
+    // (Deeper batches after the first one were measured: a long partition is bound by its arithmetic,
+    // not by the rows in flight, and the extra registers spill.)
+    constexpr int RUB = RU;
     float mx[G];
 #pragma unroll
     for (int h = 0; h < G; h++) mx[h] = -INFINITY;
-    for (int rb = 0; rb < rounds; rb += RU) {
-        if (rb > 0) {
+    auto score_round = [&](const uint4 &krow, int r) {
+        float sc[G];
+        scores_of(krow, sc);
 #pragma unroll
-            for (int u = 0; u < RU; u++) {
-                const int r = token_of(rb + u);
-                if (r < T) kraw[u] = load_kv(kbase, r);
-            }
+        for (int h = 0; h < G; h++) mx[h] = fmaxf(mx[h], sc[h]);
+        if (scores_fit && sub == 0) *(MK_LDS f32x4 *)&sm->scores[r][0] = f32x4{sc[0], sc[1], sc[2], sc[3]};
+    };
+#pragma unroll
+    for (int u = 0; u < RU; u++) {
+        const int r = token_of(u);
+        if (r < T) score_round(kraw[u], r);  // the LPT lanes of a token share r, so they are active together
+    }
+    for (int rb = RU; rb < rounds; rb += RUB) {
+        uint4 kb[RUB];
+#pragma unroll
+        for (int u = 0; u < RUB; u++) {
+            const int r = token_of(rb + u);
+            if (r < T) kb[u] = load_kv(kbase, r);
         }
 #pragma unroll
-        for (int u = 0; u < RU; u++) {
+        for (int u = 0; u < RUB; u++) {
             const int r = token_of(rb + u);
-            if (r < T) {  // the LPT lanes of a token share r, so they are active together
-                float kf[8], sc[G];
-                unpack8(kraw[u], kf);
-#pragma unroll
-                for (int h = 0; h < G; h++) {
-                    float acc = 0.0f;
-#pragma unroll
-                    for (int e = 0; e < 8; e++) acc = fmaf(q[h][e], kf[e], acc);
-                    sc[h] = group_tree_sum<LPT>(acc) * a.attn_scale;
-                    mx[h] = fmaxf(mx[h], sc[h]);
-                }
-                if (sub == 0) *(MK_LDS f32x4 *)&sm->scores[r][0] = f32x4{sc[0], sc[1], sc[2], sc[3]};
-            }
+            if (r < T) score_round(kb[u], r);
         }
     }
     trace_consumer(c, 18);
@@ -1696,7 +1710,7 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
         hm[0] = m.x; hm[1] = m.y; hm[2] = m.z; hm[3] = m.w;
     }
     // p = exp(s - max), once per (token, head), in place
-    {
+    if (scores_fit) {
         MK_LDS float *flat = &sm->scores[0][0];
         for (int i = c.tid; i < G * T; i += kConsumerThreads) {
             const int h = i & (G - 1);
@@ -1714,28 +1728,65 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
 #pragma unroll
         for (int e = 0; e < 8; e++) acc[h][e] = 0.0f;
     }
-    for (int rb = 0; rb < rounds; rb += RU) {
-        if (rb > 0) {
+    auto value_round = [&](const uint4 &vrow, const float (&p)[G]) {
+        float vf[8];
+        unpack8(vrow, vf);
 #pragma unroll
-            for (int u = 0; u < RU; u++) {
-                const int r = token_of(rb + u);
-                if (r < T) vraw[u] = load_kv(vbase, r);
-            }
+        for (int h = 0; h < G; h++) {
+            lsum[h] = lsum[h] + p[h];
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc[h][e] = fmaf(p[h], vf[e], acc[h][e]);
         }
+    };
+    if (scores_fit) {
+        auto from_buffer = [&](const uint4 &vrow, int r) {
+            const f32x4 pv = *(const MK_LDS f32x4 *)&sm->scores[r][0];
+            const float p[G] = {pv.x, pv.y, pv.z, pv.w};
+            value_round(vrow, p);
+        };
 #pragma unroll
         for (int u = 0; u < RU; u++) {
-            const int r = token_of(rb + u);
-            if (r < T) {
-                float vf[8];
-                unpack8(vraw[u], vf);
-                const f32x4 pv = *(const MK_LDS f32x4 *)&sm->scores[r][0];
-                const float p[G] = {pv.x, pv.y, pv.z, pv.w};
+            const int r = token_of(u);
+            if (r < T) from_buffer(vraw[u], r);
+        }
+        for (int rb = RU; rb < rounds; rb += RUB) {
+            uint4 vb[RUB];
 #pragma unroll
-                for (int h = 0; h < G; h++) {
-                    lsum[h] = lsum[h] + p[h];
+            for (int u = 0; u < RUB; u++) {
+                const int r = token_of(rb + u);
+                if (r < T) vb[u] = load_kv(vbase, r);
+            }
 #pragma unroll
-                    for (int e = 0; e < 8; e++) acc[h][e] = fmaf(p[h], vf[e], acc[h][e]);
+            for (int u = 0; u < RUB; u++) {
+                const int r = token_of(rb + u);
+                if (r < T) from_buffer(vb[u], r);
+            }
+        }
+    } else {
+        // the scores were not kept: the same arithmetic on the same K rows gives them again, bit for bit
+        constexpr int RUL = RU;
+        auto recomputed = [&](const uint4 &krow, const uint4 &vrow) {
+            float sc[G], p[G];
+            scores_of(krow, sc);
+#pragma unroll
+            for (int h = 0; h < G; h++) p[h] = mkm::expf_exact(sc[h] - hm[h]);
+            value_round(vrow, p);
+        };
+        // the first batch of K was consumed by pass 1 and is fetched again with the rest
+        for (int rb = 0; rb < rounds; rb += RUL) {
+            uint4 kb[RUL], vb[RUL];
+#pragma unroll
+            for (int u = 0; u < RUL; u++) {
+                const int r = token_of(rb + u);
+                if (r < T) {
+                    kb[u] = load_kv(kbase, r);
+                    vb[u] = load_kv(vbase, r);
                 }
+            }
+#pragma unroll
+            for (int u = 0; u < RUL; u++) {
+                const int r = token_of(rb + u);
+                if (r < T) recomputed(kb[u], vb[u]);
             }
         }
     }
@@ -1866,7 +1917,13 @@ static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot
                 if (leader) st_f32(a.attn_lse_intermediates + (size_t)head * MP + out_idx, r.lse);
             }
             wait_stores();
-            if (leader) signal_sharded_lane(c, layer, 2, 1);
+            // A terminal merge completes the head for the O projection (barrier row 2).  A merge
+            // inside a reduction tree is one more arrival among the head's partial results (row 1):
+            // the merge that consumes it waits for the partitions plus the merges below it.
+            if (leader) {
+                if (terminal) signal_sharded_lane(c, layer, 2, 1);
+                else add_i32(pad_ptr(c, layer, 1, head), 1);
+            }
             trace_consumer(c, 28);
             trace_consumer_flush(c, 26, 28);
         } else if (c.lane == 0) {
@@ -1908,15 +1965,6 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
         static_assert(sizeof(mk_llama_args) % 4 == 0 && sizeof(mk_llama_args) / 4 <= kThreads, "argument block");
         if (tid < (int)(sizeof(mk_llama_args) / 4)) dst[tid] = src[tid];
     }
-    // Instruction fetch (reference: controller warp, include/controller/instruction_fetch.cuh:10-27):
-    // the whole queue of this worker is copied into LDS once, so decoding an instruction never
-    // waits on HBM.
-    {
-        const int *queue = a.instructions + (size_t)blockIdx.x * a.num_slots * MK_INSTRUCTION_WORDS;
-        const int words = a.num_slots * MK_INSTRUCTION_WORDS;
-        MK_LDS int *dst = &sm->queue[0][0];
-        for (int i = tid; i < words; i += kThreads) dst[i] = queue[i];
-    }
     if (tid == 0) {
         int *const ws = static_cast<int *>(a.workspace);
         const WsLayout w = ws_layout(a.num_layers, a.hidden_size, a.intermediate_size, a.matvec_reduction_size);
@@ -1935,13 +1983,28 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
         sm->k.down_jobs = (a.intermediate_size / a.matvec_reduction_size) * (a.hidden_size / 16);
         sm->k.o_jobs = (a.hidden_size / a.matvec_reduction_size) * (a.hidden_size / 16);
     }
-    wg_barrier();
-    // decode the matvec instructions of the queue, one thread per slot
-    for (int slot = tid; slot < a.num_slots; slot += kThreads) {
-        const int opcode = sm->queue[slot][0];
-        if (opcode == 1 || (opcode >= 4 && opcode <= 6)) decode_matvec(sm, slot, a);
-    }
-    wg_barrier();
+    // Instruction fetch (reference: controller warp, include/controller/instruction_fetch.cuh:10-27):
+    // a window of the worker's queue is copied into LDS and its matvec instructions are decoded,
+    // so that taking an instruction never waits on HBM.  The usual queue fits the window and is
+    // fetched once per launch; a longer one goes through window by window, every step.
+    auto fetch_window = [&](int base) {
+        const int count = min(kQueueSlots, a.num_slots - base);
+        const int *queue = a.instructions + ((size_t)blockIdx.x * a.num_slots + base) * MK_INSTRUCTION_WORDS;
+        MK_LDS int *dst = &sm->queue[0][0];
+        for (int i = tid; i < count * MK_INSTRUCTION_WORDS; i += kThreads) dst[i] = queue[i];
+        if (tid == 0) {
+            sm->window_base = base;
+            sm->window_count = count;
+            sm->parked_slot = -1;
+        }
+        wg_barrier();
+        for (int slot = tid; slot < count; slot += kThreads) {
+            const int opcode = sm->queue[slot][0];
+            if (opcode == 1 || (opcode >= 4 && opcode <= 6)) decode_matvec(sm, slot, a);
+        }
+        wg_barrier();
+    };
+    fetch_window(0);
 
     // The handlers get the address of a kernel-local word for their refusal code.  Besides carrying
     // the code it keeps the calls from being marked as tail calls, which lets the compiler drop the
@@ -1959,7 +2022,13 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
     const WsLayout wl = ws_layout(a.num_layers, a.hidden_size, a.intermediate_size, a.matvec_reduction_size);
     int *status = static_cast<int *>(a.workspace) + wl.status;
     for (int step = 0; step < steps; step++) {
-        for (int slot = 0; slot < a.num_slots && refusal == 0; slot++) {
+      for (int base = 0; base < a.num_slots && refusal == 0; base += kQueueSlots) {
+        if (sm->window_base != base) {
+            wg_barrier();  // nobody is still reading the window that goes
+            fetch_window(base);
+        }
+        const int window_slots = min(kQueueSlots, a.num_slots - base);
+        for (int slot = 0; slot < window_slots && refusal == 0; slot++) {
             const int opcode = sm->queue[slot][0];
             if (opcode == 0) continue;  // NoOp pads the queues (megakernels/scheduler.py:287-289)
             {
@@ -1974,7 +2043,7 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
             case 3: ok = op_attention_reduction<D>(sm, slot, &refusal); break;
             case 4:
                 if constexpr (KC_HID == KC_RED && MK_PAIR_OPROJ_UPGATE) {
-                    if (slot + 1 < a.num_slots && sm->queue[slot + 1][0] == 5) {
+                    if (slot + 1 < window_slots && sm->queue[slot + 1][0] == 5) {
                         // rows can be parked when the wait is long (no attention just before, and a
                         // partition merge between attention and O-proj: with a single partition per head
                         // the wait is too short for it to pay) and the up/gate instruction is small
@@ -2006,6 +2075,8 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
             if (!ok) break;
             trace_event(make_ctx(sm, slot, sm->queue[slot][0]), kEvEnd);
         }
+        if (sm->abort) break;
+      }
         if (refusal && tid == 0) sm->abort = refusal;
 
         // End of a step.  The last workgroup to get here folds the sharded counters into `barriers`
@@ -2288,9 +2359,6 @@ int validate(const mk_llama_args &a, KernelFn *kernel) {
     // weight rows are addressed as 32-bit offsets into one buffer per matrix
     const uint64_t widest = 2ull * hid * (uint64_t)(a.vocab_size > a.intermediate_size ? a.vocab_size : a.intermediate_size);
     if (widest >= (1ull << 31)) return fail(-3, "a weight matrix of %llu bytes exceeds the 2 GiB a buffer can address", (unsigned long long)widest);
-    if (a.num_slots > kQueueSlots)
-        return fail(-3, "instruction queues have %d slots, the kernel keeps at most %d per worker in LDS", a.num_slots,
-                    kQueueSlots);
     KernelFn fn = pick_kernel(hid, R, D);
     if (!fn) return fail(-5, "no kernel instance for hidden %d, reduction width %d, head_dim %d", hid, R, D);
     const uint64_t need = mk_llama_workspace_bytes(a.num_layers, hid, a.intermediate_size, R);

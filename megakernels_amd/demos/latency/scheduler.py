@@ -29,7 +29,10 @@ Generalisations beyond the reference (which only runs Llama-3.2-1B on 132 or
 * ``num_attention_partitions > 1`` emits the split-KV schedule that the
   reference's interpreters define but its scheduler never produces
   (``:276-277``): per KV head ``P`` partial-attention instructions, then one
-  terminal reduction per group of ``attn_reduction_size`` query heads.
+  terminal reduction per group of ``attn_reduction_size`` query heads.  More
+  partitions than a reduction can list (25) go through a two-level reduction
+  tree (the reference's open TODO, ``:21-35``): non-terminal merges over runs
+  of partitions, then the terminal merge over their outputs.
 """
 
 from __future__ import annotations
@@ -63,6 +66,24 @@ def pick_num_attention_partitions(prompt_len: int, ntok: int, device=None) -> in
     min_chunk_size = 256
     num_divisions = math.ceil((prompt_len + ntok) / min_chunk_size)
     return max(1, min(num_divisions, 24))
+
+
+def reduction_tree_runs(num_partitions: int) -> list[tuple[int, int]]:
+    """How the partitions of a head are merged: one run ``[(0, P)]`` when a single merge can list them
+    all, otherwise consecutive runs of near-equal length, one first-level merge each, as few as the
+    list length allows (so the terminal merge is short)."""
+    P, cap = num_partitions, MAX_ATTENTION_PARTITIONS
+    if P <= cap:
+        return [(0, P)]
+    groups = math.ceil(P / cap)
+    bounds = [round(i * P / groups) for i in range(groups + 1)]
+    return [(bounds[i], bounds[i + 1]) for i in range(groups)]
+
+
+def reduction_tree_groups(num_partitions: int) -> int:
+    """Intermediate slots the first-level merges of a head need (0 without a tree)."""
+    runs = reduction_tree_runs(num_partitions)
+    return len(runs) if len(runs) > 1 else 0
 
 
 def make_globals(model, skip_attn_reduction: bool = True) -> Globals:
@@ -250,8 +271,10 @@ def make_dag_layer(
         assert not globs.skip_attn_reduction, (
             "a split-KV schedule needs skip_attn_reduction=False"
         )
-        assert 1 < P <= MAX_ATTENTION_PARTITIONS
-        assert P <= globs.attn_lse_intermediates.shape[1]
+        assert 1 < P <= MAX_ATTENTION_PARTITIONS * MAX_ATTENTION_PARTITIONS
+        assert P + reduction_tree_groups(P) <= globs.attn_lse_intermediates.shape[1], (
+            "the intermediate buffers hold one slot per partition and per first-level merge"
+        )
 
     new_nodes: list[DAG_Node] = []
 
@@ -302,18 +325,48 @@ def make_dag_layer(
         gqa = globs.gqa_ratio()
         group = globs.attn_reduction_size
         reduction_nodes: list[DAG_Node] = []
+        # A merge lists at most MAX_ATTENTION_PARTITIONS entries (32-word instruction).  More
+        # partitions go through a two-level tree (the reference's "TODO ... better reduction tree",
+        # ``:21-35``): first-level merges over consecutive runs of partitions, each written to a slot
+        # behind the partitions' own and counted as one more partial result of its heads, then the
+        # terminal merge over those slots, which waits for the partitions plus the first-level merges.
+        runs = reduction_tree_runs(P)
         for head_start in range(0, H, group):
             kv_heads_touched = sorted({h // gqa for h in range(head_start, head_start + group)})
-            deps = [n for kv in kv_heads_touched for n in partials_of_kv_head[kv]]
+            partials = [partials_of_kv_head[kv] for kv in kv_heads_touched]
+            if len(runs) == 1:
+                deps = [n for of_head in partials for n in of_head]
+                ins = AttentionReduction(
+                    layer_idx=layer_idx,
+                    head_start_idx=head_start,
+                    num_partials=P,
+                    is_terminal=True,
+                    reduction_list=list(range(P)),
+                    output_partial_idx=None,
+                )
+                reduction_nodes.append(DAG_Node(ins, deps))
+                continue
+            first_level: list[DAG_Node] = []
+            for k, (lo, hi) in enumerate(runs):
+                ins = AttentionReduction(
+                    layer_idx=layer_idx,
+                    head_start_idx=head_start,
+                    num_partials=P,
+                    is_terminal=False,
+                    reduction_list=list(range(lo, hi)),
+                    output_partial_idx=P + k,
+                )
+                first_level.append(DAG_Node(ins, [of_head[i] for of_head in partials for i in range(lo, hi)]))
+            new_nodes.extend(first_level)
             ins = AttentionReduction(
                 layer_idx=layer_idx,
                 head_start_idx=head_start,
-                num_partials=P,
+                num_partials=P + len(runs),
                 is_terminal=True,
-                reduction_list=list(range(P)),
+                reduction_list=[P + k for k in range(len(runs))],
                 output_partial_idx=None,
             )
-            reduction_nodes.append(DAG_Node(ins, deps))
+            reduction_nodes.append(DAG_Node(ins, first_level))
         new_nodes.extend(reduction_nodes)
         attention_outputs = reduction_nodes
         if stop_after_op == "reduction":
@@ -389,41 +442,3 @@ class LatencyScheduleBuilder(ScheduleBuilder):
             globs=cls.make_globals(model, skip_attn_reduction=schedule.globs.skip_attn_reduction),
         )
 
-
-def compute_unit_assign_to_sms(instructions: list[Instruction], sm_count: int):
-    """Assignment policy ``"cu"`` (no counterpart in the reference, whose policies are in
-    ``scheduler.py:94-271``): round robin within each run of equal opcodes, except that a layer's
-    short, latency-bound chain - attention partitions, partition merges, O projections - is spread
-    so that the O-projection blocks avoid the workers that have just run a full attention partition.
-
-    Attention partitions go to the first workers, merges to the next ones, and every O-projection
-    block to the worker that has the least of the chain so far: first the idle workers, then the
-    merge workers, then workers whose partition was the last of its head (the remainder of the
-    division into partitions, often a handful of tokens), then the others; nobody gets a second
-    block before everybody has one.  With 256 workers and 17 partitions the 128 blocks land on the
-    112 idle workers, the 8 merge workers and the 8 workers with a remainder partition.  Under round
-    robin 16 of them fall to workers that have just run a full partition; those see the O
-    projection's dependency late, behind their own weight requests, and every worker then waits for
-    them.  The linear order of the instructions, and with it every barrier count, is unchanged."""
-    from megakernels_amd.scheduler import collect_into_waves
-
-    queues: list[list[Instruction]] = [[] for _ in range(sm_count)]
-    chain_load = [0] * sm_count
-    O_PROJ, MERGE, ATTENTION, REMAINDER = 1_000_000, 1_100, 1_000, 900
-    for wave in collect_into_waves(instructions):
-        opcode = wave[0].opcode()
-        if opcode == PartialAttention.opcode():
-            chain_load = [0] * sm_count   # a new layer's chain starts
-        if opcode in (PartialAttention.opcode(), AttentionReduction.opcode(), O_ProjResidual.opcode()):
-            for ins in wave:
-                if opcode == PartialAttention.opcode():
-                    weight = REMAINDER if ins.partial_idx == ins.num_partials - 1 and ins.num_partials > 1 else ATTENTION
-                else:
-                    weight = MERGE if opcode == AttentionReduction.opcode() else O_PROJ
-                worker = min(range(sm_count), key=lambda w: (chain_load[w], w))
-                chain_load[worker] += weight
-                queues[worker].append(ins)
-        else:
-            for i, ins in enumerate(wave):
-                queues[i % sm_count].append(ins)
-    return queues

@@ -20,6 +20,9 @@ class Generator:
     def generate(self, output_tokens: Tensor, prompt_len: int, ntok: int, ntok_already_generated: int = 1):
         raise NotImplementedError
 
+    def check(self):
+        """Raise if the tokens produced so far cannot be trusted (nothing to check by default)."""
+
     def generate_with_eos(
         self,
         output_tokens: Tensor,
@@ -36,7 +39,9 @@ class Generator:
         for done in range(1, ntok, eos_token_check_interval):
             chunk = min(eos_token_check_interval, ntok - done)
             self.generate(output_tokens, prompt_len=prompt_len, ntok=chunk, ntok_already_generated=done)
-            for j, token in enumerate(output_tokens[0, done : done + chunk].cpu().tolist()):
+            tokens = output_tokens[0, done : done + chunk].cpu().tolist()  # synchronises
+            self.check()  # a chunk whose launch gave up holds garbage: raise instead of returning it
+            for j, token in enumerate(tokens):
                 if token in eos_token_ids:
                     # the first token came from prefill, hence the -1
                     return done + j, done + chunk - 1
@@ -97,6 +102,12 @@ class MK_Generator(Generator):
     def replace_with_noops(self):
         self.schedule.globs.instructions.zero_()
 
+    def check(self):
+        """Synchronise and raise if a launch since the last check gave up."""
+        check = getattr(self.interpreter, "check_status", None)
+        if check is not None and not self.skip_mk:
+            check(self.schedule.globs.barriers.device)
+
     def run(self, input_ids: Tensor, pos_id: int):
         globs = self.schedule.globs
         if not self.skip_rest:
@@ -110,7 +121,15 @@ class MK_Generator(Generator):
             return input_ids
         return torch.argmax(globs.logits, dim=-1)
 
-    def generate(self, output_tokens: Tensor, prompt_len: int, ntok: int, ntok_already_generated: int = 1):
+    def generate(self, output_tokens: Tensor, prompt_len: int, ntok: int, ntok_already_generated: int = 1,
+                 check: bool = False):
+        """``check``: synchronise at the end and raise if a launch gave up (for callers that are
+        about to read the tokens anyway; the reference's loop has no such step)."""
+        self._generate(output_tokens, prompt_len, ntok, ntok_already_generated)
+        if check:
+            self.check()
+
+    def _generate(self, output_tokens: Tensor, prompt_len: int, ntok: int, ntok_already_generated: int = 1):
         if self.fused_step and output_tokens.dtype == torch.int64 and output_tokens.is_contiguous():
             globs = self.schedule.globs
             embed = self.model.model.embed_tokens.weight

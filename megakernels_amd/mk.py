@@ -16,18 +16,32 @@ from pathlib import Path
 DEFAULT_MK_DIR = Path(__file__).parent / "csrc"
 
 
-def get_mk_func(mk_dir: Path | str | None = None):
+def get_mk_module(mk_dir: Path | str | None = None):
     mk_dir = Path(mk_dir) if mk_dir is not None else DEFAULT_MK_DIR
     path = str(mk_dir.expanduser().absolute())
     if path not in sys.path:
         sys.path.append(path)
-    module = importlib.import_module("mk_llama")
-    return module.mk_llama
+    return importlib.import_module("mk_llama")
+
+
+def get_mk_func(mk_dir: Path | str | None = None):
+    return get_mk_module(mk_dir).mk_llama
 
 
 class MK_Interpreter:
     def __init__(self, mk_dir: Path | str | None = None):
-        self.mk_func = get_mk_func(mk_dir)
+        self.mk_module = get_mk_module(mk_dir)
+        self.mk_func = self.mk_module.mk_llama
 
     def interpret(self, globs):
         raise NotImplementedError
+
+    def check_status(self, device=None):
+        """Synchronise and raise ``RuntimeError`` if the most recent launch on ``device`` gave up (a
+        dependency wait ran out, a malformed instruction, a token outside the vocabulary): its
+        outputs are then garbage.  The reference's kernel traps or hangs in these cases
+        (``include/util.cuh:38``); this one records a status that has to be looked at.  A module in
+        ``mk_dir`` without ``check_status`` is taken to report its own failures."""
+        check = getattr(self.mk_module, "check_status", None)
+        if check is not None:
+            check(device)

@@ -231,11 +231,6 @@ def assign_to_sms(
         return wave_assign_to_sms(schedule)
     if mode == "dag":
         return assign_dag_to_sms(schedule)
-    if mode == "cu":
-        # tuned for the one-workgroup-per-compute-unit kernel; lives with the latency instruction set
-        from megakernels_amd.demos.latency.scheduler import compute_unit_assign_to_sms
-
-        return compute_unit_assign_to_sms(instructions, sm_count)
     if mode == "pool":
         assert memory_fraction is not None
         return pool_assign_to_sms(instructions, sm_count, memory_fraction=memory_fraction)

@@ -290,7 +290,11 @@ static int op_attention_reduction(mk_oracle_globals *g, const int32_t *w) {
     const int32_t *list = w + 6;
     const int out_idx = w[6 + n];
     const int D = g->head_dim, R = g->attn_reduction_size;
-    if (expect_barrier(g, layer, 1, hs, P, "attention reduction")) return -1;
+    /* python_vm.py:354 asserts == num_partials.  In a reduction tree (which the reference never
+     * schedules) the counter also counts the finished merges below this one, in whatever order they
+     * ran, so the check is "at least". */
+    if (g->check_barriers && BAR(g, layer, 1, hs) < P)
+        return fail("attention reduction: barriers[%d,1,%d] is %d, expected at least %d", layer, hs, BAR(g, layer, 1, hs), P);
     if (n < 1 || 7 + n > 32) return fail("attention reduction: list of %d entries", n);
     for (int i = 0; i < n; i++)
         if (list[i] < 0 || list[i] >= g->max_partials) return fail("attention reduction: slot %d", list[i]);
@@ -308,15 +312,25 @@ static int op_attention_reduction(mk_oracle_globals *g, const int32_t *w) {
             const float *o = outs + (size_t)list[i] * D;
             for (int d = 0; d < D; d++) acc[d] = fmaf(wt, o[d], acc[d]);
         }
+        /* every listed partition empty (lse -inf: a run past the end of the sequence in a reduction
+         * tree): the formula gives NaN (-inf - -inf); the merge of nothing is defined as nothing, like
+         * an empty partition itself: zeros and -inf */
+        const int nothing = M == -INFINITY;
         if (terminal) {
-            for (int d = 0; d < D; d++) g->attn_out[h * D + d] = orc_f32_to_bf16(acc[d] / den);
+            for (int d = 0; d < D; d++) g->attn_out[h * D + d] = orc_f32_to_bf16(nothing ? 0.0f : acc[d] / den);
         } else {
             float *dst = g->attn_out_intermediates + ((size_t)h * g->max_partials + out_idx) * D;
-            for (int d = 0; d < D; d++) dst[d] = acc[d] / den;
-            g->attn_lse_intermediates[(size_t)h * g->max_partials + out_idx] = M + orc_log2f(den);
+            for (int d = 0; d < D; d++) dst[d] = nothing ? 0.0f : acc[d] / den;
+            g->attn_lse_intermediates[(size_t)h * g->max_partials + out_idx] = nothing ? -INFINITY : M + orc_log2f(den);
         }
     }
-    BAR(g, layer, 2, 0) += R;
+    /* python_vm.py:391-392 adds to row 2 after every reduction, terminal or not ("the dumb way"),
+     * which would open the O projection's barrier before a tree is done.  Here a non-terminal merge
+     * is one more arrival among its heads' partial results (row 1), and only the terminal merge
+     * completes the heads for the O projection. */
+    if (terminal) BAR(g, layer, 2, 0) += R;
+    else
+        for (int h = hs; h < hs + R; h++) BAR(g, layer, 1, h) += 1;
     return 0;
 }
 

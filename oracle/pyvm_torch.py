@@ -114,21 +114,34 @@ def partial_attention(g: Globals, ins: PartialAttention):
 
 def attention_reduction(g: Globals, ins: AttentionReduction):
     layer, h0 = ins.layer_idx, ins.head_start_idx
-    _expect(g, layer, 1, h0, ins.num_partials)
+    # the reference asserts equality (python_vm.py:354); in a reduction tree, which it never schedules,
+    # the counter also holds the finished merges below this one
+    have = int(g.barriers[layer, 1, h0])
+    assert have >= ins.num_partials, f"barriers[{layer},1,{h0}] is {have}, expected at least {ins.num_partials}"
     heads = slice(h0, h0 + g.attn_reduction_size)
     idx = torch.tensor(ins.reduction_list, dtype=torch.long)
     lses = g.attn_lse_intermediates[heads][:, idx]
     outs = g.attn_out_intermediates[heads][:, idx]
     top = lses.max(dim=-1, keepdim=True).values
-    weights = (lses - top).exp2()
+    # all listed partitions empty (possible for a run of a reduction tree past the end of the
+    # sequence): the formula gives NaN; the merge of nothing is nothing, zeros and lse -inf
+    nothing = torch.isneginf(top)
+    weights = torch.where(nothing, torch.zeros_like(lses), (lses - top).exp2())
     denom = weights.sum(dim=-1, keepdim=True)
-    merged = (outs * weights.unsqueeze(-1)).sum(dim=1) / denom
+    merged = torch.where(nothing, torch.zeros_like(outs[:, 0]), (outs * weights.unsqueeze(-1)).sum(dim=1) / denom)
     if ins.is_terminal:
         g.attn_out.view(g.num_attention_heads, -1)[heads] = merged
     else:
-        g.attn_lse_intermediates[heads, ins.output_partial_idx] = (top + denom.log2()).squeeze(-1)
+        new_lse = torch.where(nothing, top, top + denom.log2())
+        g.attn_lse_intermediates[heads, ins.output_partial_idx] = new_lse.squeeze(-1)
         g.attn_out_intermediates[heads, ins.output_partial_idx] = merged
-    g.barriers[layer, 2, 0] += g.attn_reduction_size
+    # the reference bumps row 2 after every reduction (python_vm.py:391-392), which would open the O
+    # projection's barrier before a tree is done: a non-terminal merge counts as one more partial
+    # result of its heads instead
+    if ins.is_terminal:
+        g.barriers[layer, 2, 0] += g.attn_reduction_size
+    else:
+        g.barriers[layer, 1, heads] += 1
 
 
 def _matvec_residual(mat, vec, residual, ins, R):

@@ -99,6 +99,12 @@ def test_decode_1b_slice_many_steps_split_kv_in_one_launch():
                  steps_per_launch=0)
 
 
+def test_decode_tiny_long_queue_and_reduction_tree_in_one_launch():
+    # 213 slots per worker (two windows, refetched every step) and a two-level reduction tree
+    _decode_case(config_tiny(layers=17), workers=4, prefill=20, ntok=6, partitions=2, fused=True, steps_per_launch=0)
+    _decode_case(config_tiny(), workers=48, prefill=500, ntok=6, partitions=30, max_len=1024, fused=True, steps_per_launch=0)
+
+
 def test_decode_8b_slice_all_steps_in_one_launch():
     _decode_case(config_8b_slice(layers=2), workers=256, prefill=50, ntok=4, partitions=2, fused=True, steps_per_launch=0)
 
@@ -287,6 +293,33 @@ def test_failure_in_a_launch_of_several_steps_drains_the_grid():
     assert code == 1 and opcode in (3, 4)
     assert tokens[0, 2:].tolist() == [-1, -1, -1]      # nothing after the first step was produced
     test_decode_tiny_all_steps_in_one_launch()
+
+
+def test_generator_raises_when_a_chunk_gave_up():
+    """generate_with_eos looks at the kernel's status after every chunk, and generate(check=True) at
+    its end: tokens of a launch that gave up are never handed on as text."""
+    from megakernels_amd.generators import MK_Generator
+
+    model = make_model(config_tiny())
+    fill_kv(model, upto=12)
+    schedule = build_schedule(model, 16)
+    model_gpu, schedule_gpu = mirror_to_gpu(model, schedule)
+    interp, mk_mod = _interpreter()
+    gen = MK_Generator(model_gpu, interp, schedule_gpu, fused_step=True, steps_per_launch=0)
+    tokens = torch.zeros(1, 9, dtype=torch.long, device="cuda:0")
+    tokens[0, 0] = 7
+    schedule_gpu.globs.instructions[5, 1, 0] = 77      # an opcode the kernel does not know
+    mk_mod.spin_limit_us = 20000
+    try:
+        with pytest.raises(RuntimeError, match="unknown opcode"):
+            gen.generate_with_eos(tokens, prompt_len=12, ntok=9, eos_token_check_interval=4, eos_token_ids=[1023])
+        with pytest.raises(RuntimeError, match="unknown opcode"):
+            gen.generate(tokens, prompt_len=12, ntok=4, check=True)
+    finally:
+        mk_mod.spin_limit_us = 0
+    # the failed launches left nothing behind: the repaired schedule decodes
+    schedule_gpu.globs.instructions.copy_(schedule.globs.instructions)
+    gen.generate(tokens, prompt_len=12, ntok=4, check=True)
 
 
 def test_unknown_opcode_and_bad_fields_are_reported():

@@ -137,9 +137,9 @@ def test_1b_slice_layer_started_after_the_o_projection():
     _suffix_case(config_1b_slice(layers=2), workers=256, pos=70, start_after_op="oproj")
 
 
-def _tiny_long_context():
+def _tiny_long_context(positions=8192):
     cfg = config_tiny()
-    cfg.max_position_embeddings = 8192      # length of the rotary tables
+    cfg.max_position_embeddings = positions      # length of the rotary tables
     return cfg
 
 
@@ -148,25 +148,39 @@ def test_tiny_partition_of_exactly_the_on_chip_limit():
     _one_step_case(_tiny_long_context(), workers=16, pos=4095, max_len=4096 + 8)
 
 
-def test_partition_beyond_the_on_chip_limit_is_reported():
+def test_single_partition_beyond_the_score_buffer():
+    """The reference's own schedule has one partition per KV head whatever the context length
+    (demos/latency/scheduler.py:276-277, max_len_override=16384 in scripts/generate.py:43) and its
+    kernel walks it block by block (attention_partial.cu:463-520).  Here a partition of more than 4096
+    positions does not fit the on-chip score buffer and takes the path that recomputes the scores in
+    its second pass: same bits."""
+    _one_step_case(_tiny_long_context(), workers=16, pos=4100, max_len=4096 + 64)
+    _one_step_case(_tiny_long_context(16448), workers=16, pos=16384, max_len=16384 + 64)
+
+
+def test_1b_slice_single_partition_long_context():
+    _one_step_case(config_1b_slice(layers=1), workers=256, pos=5000, partitions=1, max_len=5120)
+
+
+def test_8b_slice_long_partitions():
+    # head_dim 128: two partitions of 3008 and 2993 positions (deep batches), then one of 6001 (recomputed)
+    _one_step_case(config_8b_slice(), workers=256, pos=6000, partitions=2, max_len=6144)
+    _one_step_case(config_8b_slice(), workers=256, pos=6000, partitions=1, max_len=6144)
+
+
+def test_reduction_tree():
+    """More partitions than one merge can list (25): first-level merges, then the terminal one."""
+    _one_step_case(config_tiny(), workers=64, pos=600, partitions=32, max_len=1024)
+    # 65 KV blocks over 64 partitions of two blocks: partitions 33..63 are empty, and so is the whole
+    # last run of first-level merges
+    _one_step_case(_tiny_long_context(), workers=96, pos=1029, partitions=64, max_len=1100)
+    _one_step_case(config_1b_slice(layers=2), workers=256, pos=3000, partitions=40, max_len=3072)
+
+
+def test_queue_longer_than_the_on_chip_window():
+    """20 layers on 4 workers: 260 instructions per worker go through the 192-slot window in two
+    fetches (the reference streams instructions from global memory, include/controller/instruction_fetch.cuh:10-27)."""
     import sys
 
-    cfg = _tiny_long_context()
-    model = make_model(cfg, max_len=4096 + 64)
-    fill_kv(model, upto=4100)
-    schedule = build_schedule(model, 16)
-    schedule.globs.pos_id = 4100                       # 4101 positions in one partition
-    _, schedule_gpu = mirror_to_gpu(model, schedule)
-    from megakernels_amd.demos.latency.mk import LatencyMK_Interpreter
-
-    mk_mod_interp = LatencyMK_Interpreter()
-    mk_mod = sys.modules["mk_llama"]
-    mk_mod.spin_limit_us = 20000
-    try:
-        mk_mod_interp.interpret(schedule_gpu.globs)
-        code, worker, slot, opcode = mk_mod.read_status("cuda:0")
-    finally:
-        mk_mod.spin_limit_us = 0
-    assert code == 3 and opcode == 2
-    # and the same context split in two partitions is fine
-    _one_step_case(cfg, workers=16, pos=4100, partitions=2, max_len=4096 + 64)
+    cfg = config_tiny(layers=20)
+    _one_step_case(cfg, workers=4, pos=33, partitions=2)

@@ -260,6 +260,50 @@ def test_split_kv_equals_single_partition():
         assert np.abs(merged - want_lse).max() <= lse_tol
 
 
+@pytest.mark.parametrize("P", [32, 64])
+def test_reduction_tree_equals_single_partition(P):
+    """A whole layer's attention through a two-level reduction tree (P partitions, first-level merges,
+    terminal merge) reproduces the unsplit softmax, and leaves the counters in their closed form:
+    row 1 holds the partitions plus the first-level merges of each head, row 2 the heads."""
+    from megakernels_amd.demos.latency.scheduler import reduction_tree_runs
+
+    cfg = config_tiny()
+    pos = 16 * P + 5                      # every partition has tokens, the last one five
+
+    def fresh(*args, **kw):
+        # the newest position is normally written by the QKV instruction, which this test leaves out
+        model, sched, g = globals()["fresh"](*args, **kw)
+        row = torch.Generator().manual_seed(9)
+        for cache in model.stacked_kv_cache:
+            cache[:, :, pos] = torch.randn(cache[:, :, pos].shape, generator=row).to(cache.dtype)
+        return model, sched, g
+
+    model, sched, g = fresh(cfg, workers=96, pos=pos, partitions=1)
+    gen = torch.Generator().manual_seed(6)
+    g.post_ln_rope_q.copy_(torch.randn(g.post_ln_rope_q.shape, generator=gen).to(torch.bfloat16))
+    want = [_attention_ref(g, 1, kv, 0, pos + 1)[0] for kv in range(cfg.num_key_value_heads)]
+    model2, sched2, g2 = fresh(cfg, workers=96, pos=pos, partitions=P)
+    g2.post_ln_rope_q.copy_(g.post_ln_rope_q)
+    g2.barriers[1, 0] = 4
+    chain = [i for i in sched2.get_linear_instructions() if i.opcode() in (2, 3) and i.layer_idx == 1]
+    pyvm.interpret(g2, chain)
+    got = f64(g2.attn_out).reshape(cfg.num_attention_heads, -1)
+    for kv in range(cfg.num_key_value_heads):
+        ref = want[kv]
+        assert np.abs(got[4 * kv : 4 * kv + 4] - bf16_round(ref)).max() <= BF16_EPS * np.abs(ref).max() * 1.01
+    runs = reduction_tree_runs(P)
+    assert len(runs) > 1
+    assert (g2.barriers[1, 1, : cfg.num_attention_heads] == P + len(runs)).all()
+    assert int(g2.barriers[1, 2, 0]) == cfg.num_attention_heads
+    # the torch restatement agrees on the counters and, within rounding, on the result
+    model3, sched3, g3 = fresh(cfg, workers=96, pos=pos, partitions=P)
+    g3.post_ln_rope_q.copy_(g.post_ln_rope_q)
+    g3.barriers[1, 0] = 4
+    pyvm_torch.interpret(g3, [i for i in sched3.get_linear_instructions() if i.opcode() in (2, 3) and i.layer_idx == 1])
+    assert torch.equal(g3.barriers, g2.barriers)
+    assert np.abs(f64(g3.attn_out) - f64(g2.attn_out)).max() <= 2e-2 * np.abs(f64(g2.attn_out)).max()
+
+
 def test_attention_reduction_nonterminal_and_list_order():
     cfg = config_tiny()
     model, sched, g = fresh(cfg, pos=100, partitions=4)

@@ -205,7 +205,36 @@ def test_split_kv_schedule():
     assert kinds.index(3) > max(j for j, k in enumerate(kinds) if k == 2)
     assert kinds.index(4) > max(j for j, k in enumerate(kinds) if k == 3)
     with pytest.raises(AssertionError):
-        build(cfg_1b(1), 256, num_attention_partitions=MAX_ATTENTION_PARTITIONS + 1)
+        build(cfg_1b(1), 256, num_attention_partitions=MAX_ATTENTION_PARTITIONS * MAX_ATTENTION_PARTITIONS + 1)
+    with pytest.raises(AssertionError):          # 250 partitions + 10 first-level merges need 260 slots
+        build(cfg_1b(1), 256, num_attention_partitions=250)
     assert pick_num_attention_partitions(4096, 64) == 17
     assert pick_num_attention_partitions(32, 128) == 1
     assert pick_num_attention_partitions(16384, 64) == 24
+
+
+@pytest.mark.parametrize("P", [26, 32, 64])
+def test_reduction_tree_schedule(P):
+    """More partitions than one reduction can list: first-level merges over consecutive runs, written
+    behind the partitions' slots, then one terminal merge over their outputs that waits for the
+    partitions plus the first-level merges (the reference's open TODO, demos/latency/scheduler.py:21-35)."""
+    from megakernels_amd.demos.latency.scheduler import reduction_tree_runs
+
+    sched = build(cfg_1b(1), 256, num_attention_partitions=P)
+    ins = sched.get_linear_instructions()
+    runs = reduction_tree_runs(P)
+    assert len(runs) == -(-P // MAX_ATTENTION_PARTITIONS) and runs[0][0] == 0 and runs[-1][1] == P
+    assert all(a[1] == b[0] for a, b in zip(runs, runs[1:])) and max(hi - lo for lo, hi in runs) <= MAX_ATTENTION_PARTITIONS
+    reds = [i for i in ins if i.opcode() == 3]
+    assert len(reds) == 8 * (len(runs) + 1)
+    for head_start in range(0, 32, 4):
+        mine = [i for i in reds if i.head_start_idx == head_start]
+        first, last = mine[:-1], mine[-1]
+        assert [tuple(i.reduction_list[k] for k in (0, -1)) for i in first] == [(lo, hi - 1) for lo, hi in runs]
+        assert all(not i.is_terminal and i.num_partials == P and i.output_partial_idx == P + k for k, i in enumerate(first))
+        assert last.is_terminal and last.num_partials == P + len(runs) and last.reduction_list == [P + k for k in range(len(runs))]
+    # every instruction still fits the 32-word format, and the DAG orders merges after what they read
+    from megakernels_amd.scheduler import serialize_and_pad
+    assert all(len(serialize_and_pad(i)) == 32 for i in reds)
+    kinds = [i.opcode() for i in ins]
+    assert kinds.index(4) > max(j for j, k in enumerate(kinds) if k == 3)
