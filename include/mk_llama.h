@@ -130,7 +130,10 @@ typedef struct mk_llama_args {
 } mk_llama_args;
 
 /* Bytes of scratch device memory a launch needs for these shapes.  The caller
- * zeroes it once; the kernel leaves it clean after every successful launch.
+ * zeroes it once; the kernel leaves it usable for the next launch after every
+ * successful one (counters back at zero; a count of completed decode steps and
+ * tagged partial sums stay, and later launches rely on both - do not share a
+ * workspace between models, and zero it again after a launch that gave up).
  * Holds sharded barrier counters, residual partial sums and the status block. */
 uint64_t mk_llama_workspace_bytes(int32_t num_layers, int32_t hidden_size, int32_t intermediate_size,
                                   int32_t matvec_reduction_size);
@@ -146,7 +149,7 @@ int mk_llama_launch(const mk_llama_args *args, void *hip_stream);
  * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No
  * counterpart in the reference.  `args->workspace` and `args->workspace_bytes` are ignored; the
  * workspace is an array inside the library (2 MiB per GPU, held until the process ends), which is
- * enough for every shape the kernel has an instance for (1B: 250 KB, 8B with 32 layers: 950 KB).
+ * enough for every shape the kernel has an instance for (1B: 280 KB, 8B with 32 layers: 1.01 MiB).
  * Shapes that need more are refused with -6 and a message.  The call allocates nothing: it zeroes
  * the part of the array it is going to use with a small kernel on `hip_stream`, then launches as
  * mk_llama_launch does.  `*scratch_out` (may be NULL) receives the array's device address, which is

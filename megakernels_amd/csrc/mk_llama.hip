@@ -27,6 +27,10 @@
 //     as 16 shards in the workspace while the kernel runs (256 atomics on one address cost
 //     ~3 us, 16 per shard ~0.2 us); the last workgroup to finish adds the shard totals into
 //     `barriers`, so after the launch the tensor holds exactly the reference VM's counts.
+//   * a residual projection over several column groups (down; O-proj of 4096-wide models) leaves
+//     the groups' partial sums as (value, tag) pairs in the workspace; the job of the last group
+//     fetches them until every tag is the current phase's and applies them in group order, the
+//     Python VM's order, so the bf16 rounding chain is reproduced without serialising the workers.
 //   * every barrier wait is bounded (spin_limit_us): on expiry the worker records a status
 //     code and every workgroup leaves its instruction loop, so the grid always drains.
 //   * optionally the per-token glue of the reference's decode loop is part of the launch (embedding
@@ -76,6 +80,7 @@ constexpr int kGqa = 4;             // query heads per KV head handled by one at
 constexpr int kStatusInts = 16;
 constexpr int kDoneSlot = 8;        // workspace int: workgroups finished, summed over the steps of a launch
 constexpr int kStepSlot = 9;        // workspace int: decode steps of this launch completed and published
+constexpr int kEpochSlot = 10;      // workspace int: decode steps completed since the workspace was zeroed
 
 // Weight rows in flight per consumer wave, per instruction kind (16 VGPRs per 2048-element row; the
 // 9-wave workgroup leaves each lane 168 VGPRs).  The rows requested before the dependency wait are
@@ -123,7 +128,7 @@ constexpr int rows_in_flight(int wanted) { return KC <= 4 ? wanted : (wanted < M
 // workspace layout (ints unless noted)
 // ---------------------------------------------------------------------------------------------
 struct WsLayout {
-    size_t status, shards, arrive_o, arrive_d, argmax, partial, pads, total_bytes;
+    size_t status, shards, argmax, partial, pads, total_bytes;
 };
 constexpr int kMaxWorkers = 1024;   // workers that can report an LM-head maximum
 constexpr int kPadInts = 32;        // a padded counter owns a 128-byte line
@@ -137,13 +142,11 @@ __host__ __device__ inline WsLayout ws_layout(int L, int hid, int inter, int R) 
     w.status = off;   off += kStatusInts;
     off = (off + 31) & ~(size_t)31;  // counters start on a 128-byte line
     w.shards = off;   off += (size_t)kReplicas * kShards * L * kHotRows;
-    w.arrive_o = off; off += hid / 16;
-    w.arrive_d = off; off += hid / 16;
     w.argmax = off;   off += 2 * (size_t)kMaxWorkers;  // per worker: value bits, index + 1 (0: nothing)
     off = (off + 3) & ~(size_t)3;
-    w.partial = off;  // floats: [max(groups_o, groups_d)][hid]
+    w.partial = off;  // (value, tag) pairs of 8 bytes: [max(groups_o, groups_d)][hid]
     int g_o = hid / R, g_d = inter / R;
-    off += (size_t)(g_o > g_d ? g_o : g_d) * hid;
+    off += (size_t)(g_o > g_d ? g_o : g_d) * hid * 2;
     // the per-head counters (barrier rows 0 and 1), one cache line each
     off = (off + 31) & ~(size_t)31;
     w.pads = off;     off += (size_t)L * 2 * pad_cols(hid) * kPadInts;
@@ -156,8 +159,9 @@ __host__ __device__ inline WsLayout ws_layout(int L, int hid, int inter, int R) 
 // ---------------------------------------------------------------------------------------------
 // What every instruction needs and no instruction changes: computed once per launch, read from LDS.
 struct Consts {
-    int *status, *shards, *arrive_o, *arrive_d, *argmax, *pads;  // regions of the workspace
-    float *partial;
+    int *status, *shards, *argmax, *pads;  // regions of the workspace
+    uint64_t *partial;              // residual partial sums as (value, tag) pairs
+    uint32_t epoch;                 // decode steps completed in this workspace before the current one
     int *trace_base;                // this worker's rows of `timings`, or nullptr when tracing is off
     long long spin_ticks;           // limit of a dependency wait, in wall-clock ticks
     int cols;                       // columns of `barriers`: query + key + value heads
@@ -181,7 +185,7 @@ struct Smem {
     int window_base, window_count;  // which slots of the worker's queue are in `queue` / `desc`: [base, base + count)
     Consts k;
     mk_llama_args args;             // the launch arguments, read from here by every instruction
-    int flags[kOutRows / 16];       // per-block "I was the last arriver" (matvec-add)
+    int flags[16];                  // scratch of the end-of-step reduction
 #ifdef MK_TRACE_CONSUMER
     int consumer_ticks[16];         // development trace: consumer timestamps parked until the instruction ends
 #endif
@@ -432,8 +436,7 @@ __device__ __forceinline__ Ctx make_ctx(SmemPtr sm, int slot, int opcode) {
 // workspace regions
 __device__ __forceinline__ int *ws_status(const Ctx &c) { return uni(c.sm->k.status); }
 __device__ __forceinline__ int *ws_shards(const Ctx &c) { return uni(c.sm->k.shards); }
-__device__ __forceinline__ int *ws_arrive(const Ctx &c, bool down) { return uni(down ? c.sm->k.arrive_d : c.sm->k.arrive_o); }
-__device__ __forceinline__ float *ws_partial(const Ctx &c) { return uni(c.sm->k.partial); }
+__device__ __forceinline__ uint64_t *ws_partial(const Ctx &c) { return uni(c.sm->k.partial); }
 __device__ __forceinline__ long long spin_ticks(const Ctx &c) {
     const long long v = c.sm->k.spin_ticks;
     return ((long long)uni((int)(v >> 32)) << 32) | (uint32_t)uni((int)v);
@@ -1017,13 +1020,20 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
         });
 }
 
+// Tag of the residual partial sums of one (decode step, layer, projection): differs from whatever a
+// slot of the partial-sum buffer held before (the previous projection that used the group, or zero).
+__device__ __forceinline__ uint32_t phase_tag(const Ctx &c, int layer, bool is_down) {
+    const uint32_t step = (uint32_t)uni((int)c.sm->k.epoch);
+    const uint32_t tag = (step * (uint32_t)uni(c.sm->args.num_layers) + (uint32_t)layer) * 2u + (is_down ? 1u : 0u) + 1u;
+    return tag ? tag : 1u;
+}
+
 // ---------------------------------------------------------------------------------------------
 // opcodes 4 and 6: matvec over one column group + residual add  (python_vm.py:59-124;
 // reference device op: demos/low-latency-llama/matvec_adds.cu:10-192).
-// With several column groups each (group, block) job parks its bf16-rounded partial in the
-// workspace; the job that arrives last on the block's counter applies the partials to the
-// residual in group order, which is the order the Python VM applies them in, so the bf16
-// rounding chain is reproduced without serialising the workers.
+// With several column groups each (group, block) job leaves its bf16-rounded partial sum in the
+// workspace as a tagged pair, and the job of the last group applies them to the residual in group
+// order, which is the order the Python VM applies them in.
 // ---------------------------------------------------------------------------------------------
 template <int KC, bool is_down>
 __device__ __forceinline__ bool control_matvec_add(const Ctx &c) {
@@ -1068,6 +1078,7 @@ __device__ __forceinline__ bool control_matvec_add(const Ctx &c) {
             }
         },
         [&]() {
+            bool guards_data = true;
             if (ngroups == 1) {
                 for (int p = c.lane; p < nblk * 8; p += 64) {
                     const int row0 = start * 16 + p * 2;
@@ -1077,46 +1088,63 @@ __device__ __forceinline__ bool control_matvec_add(const Ctx &c) {
                     st_u32(resid + row0, mkm::pack_bf16(lo, hi));
                 }
             } else {
-                int *arrive = ws_arrive(c, is_down);
-                float *partial = ws_partial(c);
-                for (int t = c.lane; t < nblk * 16; t += 64)
-                    st_f32(partial + (size_t)group * hid + start * 16 + t, c.sm->out[t]);
-                wait_stores();
-                for (int b = c.lane; b < nblk; b += 64) {
-                    const int old = add_ret_i32(&arrive[start + b], 1);
-                    const int last = old == ngroups - 1;
-                    if (last) st_i32(&arrive[start + b], 0);
-                    c.sm->flags[b] = last;
-                }
-                compiler_fence();  // same wave: LDS operations execute in order
-                for (int p = c.lane; p < nblk * 8; p += 64) {
-                    if (!c.sm->flags[p >> 3]) continue;
-                    const int row0 = start * 16 + p * 2;
-                    const uint32_t h = prefetched ? (p < 64 ? pre[0] : pre[1]) : ld_u32(resid + row0);
-                    float lo = mkm::bf16_lo(h), hi = mkm::bf16_hi(h);
-                    auto apply = [&](uint64_t v) {
-                        lo = mkm::round_bf16(lo + mkm::bits_f32((uint32_t)v));
-                        hi = mkm::round_bf16(hi + mkm::bits_f32((uint32_t)(v >> 32)));
-                    };
-                    // The partials are applied in group order, but requested four (then two) at a time:
-                    // this worker is the one the next layer is waiting for, and a loop over the
-                    // groups would pay one round trip per group.
-                    const float *mine = partial + row0;
-                    int g = 0;
-                    for (; g + 4 <= ngroups; g += 4) {
-                        const uint64_t v0 = ld_u64(mine + (size_t)g * hid), v1 = ld_u64(mine + (size_t)(g + 1) * hid);
-                        const uint64_t v2 = ld_u64(mine + (size_t)(g + 2) * hid), v3 = ld_u64(mine + (size_t)(g + 3) * hid);
-                        apply(v0); apply(v1); apply(v2); apply(v3);
+                // Several column groups per block.  Every group's job but the last leaves its
+                // bf16-rounded sum as a (value, tag) pair - one 8-byte store, so whoever sees the tag
+                // sees the value, and nothing has to be acknowledged or counted.  The job of the last
+                // group fetches the others' pairs until all carry this phase's tag and applies them
+                // in group order, its own last: the Python VM's order.
+                uint64_t *partial = ws_partial(c);
+                const uint32_t tag = phase_tag(c, layer, is_down);
+                if (group != ngroups - 1) {
+                    for (int t = c.lane; t < nblk * 16; t += 64)
+                        st_u64(partial + (size_t)group * hid + start * 16 + t, ((uint64_t)tag << 32) | mkm::f32_bits(c.sm->out[t]));
+                    guards_data = false;
+                } else {
+                    const long long t0 = wall_clock64();
+                    const long long limit = spin_ticks(c);
+                    for (int p0 = 0; p0 < nblk * 8; p0 += 64) {  // wave-uniform trip count
+                        const int p = p0 + c.lane;
+                        const bool active = p < nblk * 8;
+                        const int row0 = start * 16 + (active ? p : 0) * 2;
+                        const uint32_t h = prefetched ? (p < 64 ? pre[0] : pre[1]) : (active ? ld_u32(resid + row0) : 0u);
+                        float lo = mkm::bf16_lo(h), hi = mkm::bf16_hi(h);
+                        const uint64_t *theirs = partial + row0;
+                        // four groups' pairs per round trip
+                        for (int g0 = 0; g0 < ngroups - 1; g0 += 4) {
+                            uint4 v[4];
+                            while (true) {
+                                bool complete = true;
+#pragma unroll
+                                for (int k = 0; k < 4; k++)
+                                    if (g0 + k < ngroups - 1) {
+                                        v[k] = active ? ld_b128(theirs + (size_t)(g0 + k) * hid) : make_uint4(0, tag, 0, tag);
+                                        complete &= v[k].y == tag && v[k].w == tag;
+                                    }
+                                if (__all(complete)) break;
+                                if (wall_clock64() - t0 > limit || ld_i32(ws_status(c)) != 0) {
+                                    if (c.lane == 0) record_status(c, MK_STATUS_BARRIER_TIMEOUT);
+                                    break;
+                                }
+                                __builtin_amdgcn_s_sleep(2);
+                            }
+#pragma unroll
+                            for (int k = 0; k < 4; k++)
+                                if (g0 + k < ngroups - 1) {
+                                    lo = mkm::round_bf16(lo + mkm::bits_f32(v[k].x));
+                                    hi = mkm::round_bf16(hi + mkm::bits_f32(v[k].z));
+                                }
+                        }
+                        if (active) {
+                            lo = mkm::round_bf16(lo + c.sm->out[p * 2]);
+                            hi = mkm::round_bf16(hi + c.sm->out[p * 2 + 1]);
+                            st_u32(resid + row0, mkm::pack_bf16(lo, hi));
+                        }
                     }
-                    for (; g + 2 <= ngroups; g += 2) {
-                        const uint64_t v0 = ld_u64(mine + (size_t)g * hid), v1 = ld_u64(mine + (size_t)(g + 1) * hid);
-                        apply(v0); apply(v1);
-                    }
-                    if (g < ngroups) apply(ld_u64(mine + (size_t)g * hid));
-                    st_u32(resid + row0, mkm::pack_bf16(lo, hi));
                 }
             }
-            wait_stores();
+            // an arrival that stands for nothing another worker reads (a partial sum carries its own
+            // tag) need not wait for its stores
+            if (guards_data) wait_stores();
             signal_sharded(c, layer, is_down ? 5 : 3, nblk);
         });
 }
@@ -1970,11 +1998,10 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
         const WsLayout w = ws_layout(a.num_layers, a.hidden_size, a.intermediate_size, a.matvec_reduction_size);
         sm->k.status = ws + w.status;
         sm->k.shards = ws + w.shards;
-        sm->k.arrive_o = ws + w.arrive_o;
-        sm->k.arrive_d = ws + w.arrive_d;
         sm->k.argmax = ws + w.argmax;
         sm->k.pads = ws + w.pads;
-        sm->k.partial = reinterpret_cast<float *>(ws + w.partial);
+        sm->k.partial = reinterpret_cast<uint64_t *>(ws + w.partial);
+        sm->k.epoch = (uint32_t)ld_i32(ws + w.status + kEpochSlot);
         sm->k.trace_base =
             (a.flags & MK_FLAG_TIMINGS) && a.timings ? a.timings + (size_t)blockIdx.x * a.num_slots * MK_TIMING_SLOTS : nullptr;
         sm->k.spin_ticks = (long long)(a.spin_limit_us ? a.spin_limit_us : 2000000u) * 100;  // 100 MHz wall clock
@@ -2185,6 +2212,7 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
                     sm->token = token;
                 }
             }
+            if (tid == 0) st_i32(&status[kEpochSlot], (int)(sm->k.epoch + 1u));
             if (more) {
                 // everything the next step relies on (zeroed counters, the token) has landed before
                 // the step is published
@@ -2225,6 +2253,7 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
         if (!more) break;
         if (tid == 0) {
             sm->args.pos_id = a.pos_id + step + 1;
+            sm->k.epoch += 1u;
             sm->parked_slot = -1;
         }
         wg_barrier();

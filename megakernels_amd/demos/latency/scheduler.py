@@ -61,11 +61,17 @@ from megakernels_amd.utils import assert_div, get_sm_count
 MAX_ATTENTION_PARTITIONS = INTS_PER_INSTRUCTION - 7
 
 
-def pick_num_attention_partitions(prompt_len: int, ntok: int, device=None) -> int:
-    """One partition per 256 cached positions, at most 24 (reference ``:21-35``)."""
+def pick_num_attention_partitions(prompt_len: int, ntok: int, device=None, num_kv_heads: int | None = None) -> int:
+    """One partition per 256 cached positions, at most 24 (reference ``:21-35``) - or, when the number
+    of KV heads is given, at most one partition per worker for every KV head if that is more (256
+    workers, 8 KV heads: 32): beyond 25 partitions the merges go through a reduction tree, which costs
+    a few microseconds per layer and pays once the partitions are long (16384 positions and up)."""
     min_chunk_size = 256
     num_divisions = math.ceil((prompt_len + ntok) / min_chunk_size)
-    return max(1, min(num_divisions, 24))
+    most = 24
+    if num_kv_heads:
+        most = max(most, get_sm_count(device if device is not None else "cuda") // num_kv_heads)
+    return max(1, min(num_divisions, most))
 
 
 def reduction_tree_runs(num_partitions: int) -> list[tuple[int, int]]:

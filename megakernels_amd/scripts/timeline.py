@@ -8,8 +8,9 @@ with seeded noise, runs a few warm-up steps, then one step with ``MK_FLAG_TIMING
 per instruction kind, how long the workers waited for the dependency, loaded the activation vector,
 computed and wrote back; and for one layer when each kind started, saw its dependency and ended across
 the workers.  ``out=`` saves the raw records (``timings`` [workers, slots, 128] and ``instructions``
-[workers, slots, 32], plain ``numpy`` arrays) for a Gantt view elsewhere - the counterpart of the
-reference's ``diff_test.py outfile=`` dump (``scripts/diff_test.py:231-242``).  The reference records the
+[workers, slots, 32], plain ``numpy`` arrays, plus ``reference_layout``: the same records in the
+reference's event slots, ``include/util.cuh:215-246``) for a Gantt view elsewhere; the dump shaped like the
+reference's ``diff_test.py outfile=`` (``scripts/diff_test.py:231-242``) comes from ``tests/diff_test.py outfile=``.  The reference records the
 same events (``include/util.cuh:215-246``) when compiled with ``TIMING_RECORD_ENABLED``; here the records
 are taken on request at run time.
 
@@ -32,6 +33,59 @@ from megakernels_amd.scheduler import assign_to_sms, tensorize_instructions
 from megakernels_amd.utils import get_sm_count, set_sm_count_override
 
 NAMES = {1: "qkv", 2: "attention", 3: "merge", 4: "o-proj", 5: "up/gate", 6: "down", 7: "lm-head"}
+
+# The reference's event slots (include/util.cuh:215-246) and the record of this kernel (MK_TIMING_* of
+# include/mk_llama.h: 0 start, 1 dependency seen, 2 input ready, 3 rows done, 4 end) each one is taken
+# from.  The reference's stages that this kernel does not have (instruction fetch, page allocation,
+# semaphore set-up: all done before an instruction starts here) get the start time.
+REFERENCE_EVENTS = {
+    0: 0,    # TEVENT_CONTROLLER_START
+    1: 0,    # TEVENT_IFETCH_DONE
+    2: 0,    # TEVENT_PAGE_ALLOC_DONE
+    3: 0,    # TEVENT_SEMS_SETUP
+    4: 4,    # TEVENT_CONTROLLER_END
+    5: 0,    # TEVENT_LOADER_START: the first weight rows are requested on entry
+    7: 2,    # TEVENT_LAUNCHER_START
+    9: 3,    # TEVENT_STORER_START
+    11: 2,   # TEVENT_CONSUMER_START
+    44: 0,   # TEVENT_AT_GMEM_WAIT
+    45: 1,   # TEVENT_DONE_GMEM_WAIT
+    46: 3,   # TEVENT_AT_GMEM_STORE
+    47: 4,   # TEVENT_DONE_GMEM_STORE
+    48: 0,   # TEVENT_FIRST_LOAD
+    49: 2,   # TEVENT_FIRST_USE
+    50: 3,   # TEVENT_FIRST_STORE
+    51: 3,   # TEVENT_LAST_LOAD
+    52: 3,   # TEVENT_LAST_USE
+    53: 4,   # TEVENT_LAST_STORE
+    54: 4,   # TEVENT_OUTPUT_READY
+}
+
+
+def launch_origin(starts) -> int:
+    """The earliest of the 32-bit clock values ``starts`` (a 1-D integer tensor or array), when they lie
+    within half the clock's range of each other - also if the clock wrapped in between."""
+    v = np.asarray(starts).astype(np.int64) & 0xFFFFFFFF
+    first = int(v[0])
+    signed = ((v - first + (1 << 31)) % (1 << 32)) - (1 << 31)
+    return (first + int(signed.min())) % (1 << 32)
+
+
+def reference_event_layout(timings: torch.Tensor, instructions: torch.Tensor) -> torch.Tensor:
+    """``timings [workers, slots, 128]`` of this kernel re-laid as the reference's tools expect them:
+    the slots of ``REFERENCE_EVENTS`` filled, as ticks (10 ns) since the first instruction of the
+    launch started; everything else zero, as are the rows of NoOp padding."""
+    t = timings.cpu().to(torch.int64)
+    ins = instructions.cpu()
+    executed = ins[:, :, 0] != 0
+    out = torch.zeros_like(t)
+    if not bool(executed.any()):
+        return out.to(torch.int32)
+    origin = launch_origin(t[:, :, 0][executed].numpy())
+    ticks = ((t[:, :, :5] & 0xFFFFFFFF) - origin) % (1 << 32)
+    for slot, source in REFERENCE_EVENTS.items():
+        out[:, :, slot] = torch.where(executed, ticks[:, :, source], torch.zeros_like(ticks[:, :, source]))
+    return out.to(torch.int32)
 
 
 def main(argv):
@@ -58,7 +112,7 @@ def main(argv):
     model = model.to(device)
     workers = get_sm_count(device)
     set_sm_count_override(workers)
-    partitions = opts["partitions"] or pick_num_attention_partitions(pos, 1)
+    partitions = opts["partitions"] or pick_num_attention_partitions(pos, 1, device, cfg.num_key_value_heads)
     schedule = LatencyScheduleBuilder.build(model, num_attention_partitions=partitions)
     tensorize_instructions(schedule.globs, assign_to_sms(opts["sched"], schedule=schedule))
     globs = schedule.globs
@@ -86,10 +140,11 @@ def main(argv):
     ins = globs.instructions.cpu().numpy()
     # the records are the low 32 bits of the device clock: times since the earliest record
     executed = t[:, :, 5] != 0
-    origin = np.int64(globs.timings.cpu()[:, :, 0].numpy()[executed].astype(np.uint32).min())
+    origin = np.int64(launch_origin(globs.timings.cpu()[:, :, 0].numpy()[executed]))
     t[:, :, :5] = ((t[:, :, :5].astype(np.int64) - origin) % (1 << 32)) / 100.0
     if opts["out"]:
         np.savez_compressed(opts["out"], timings=globs.timings.cpu().numpy(), instructions=ins,
+                            reference_layout=reference_event_layout(globs.timings, globs.instructions).numpy(),
                             ticks_per_microsecond=np.array(100))
     print(f"{opts['model']}, {opts['layers']} layers, position {pos}, {partitions} attention partitions, {workers} workers, "
           f"assignment {opts['sched']}: kernel {start.elapsed_time(end) * 1e3:.1f} us with timing records on, "

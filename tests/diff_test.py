@@ -41,6 +41,7 @@ class ScriptConfig:
     num_attention_partitions: int = 1
     barrier_init_val: int = 0
     noops: bool = False
+    outfile: str | None = None
 
     def full(self):
         self.layer_limit = None
@@ -58,6 +59,8 @@ def parse(argv):
             setattr(cfg, key, None)
         elif isinstance(current, bool):
             setattr(cfg, key, value.lower() in ("1", "true"))
+        elif key == "outfile":
+            setattr(cfg, key, value)
         elif isinstance(current, int) or key in ("layer_limit",):
             setattr(cfg, key, int(value))
         else:
@@ -106,13 +109,42 @@ def main(config: ScriptConfig):
         instructions = []
     pyvm.interpret(g, instructions, check_barriers=config.barrier_init_val == 0)
     interp = LatencyMK_Interpreter()
-    interp.interpret(schedule_gpu.globs)
-    sys.modules["mk_llama"].check_status("cuda:0")
+    mk_mod = sys.modules["mk_llama"]
+    mk_mod.record_timings = config.outfile is not None
+    try:
+        interp.interpret(schedule_gpu.globs)
+        mk_mod.check_status("cuda:0")
+    finally:
+        mk_mod.record_timings = False
     print("done! diffing tensors:")
     g.diff(schedule_gpu.globs.__class__(**{f.name: (getattr(schedule_gpu.globs, f.name).cpu()
            if isinstance(getattr(schedule_gpu.globs, f.name), torch.Tensor) else getattr(schedule_gpu.globs, f.name))
            for f in fields(schedule_gpu.globs)}))
     print("elements that differ bit for bit:", mismatches(g, schedule_gpu.globs) or "none")
+    if config.outfile is not None:
+        # the reference's dump (scripts/diff_test.py:231-242): timings, instruction words, the
+        # instruction objects per worker and the summed cost per worker.  `timings` is in the
+        # reference's event slots (include/util.cuh:215-246); `timings_native` as the kernel wrote them.
+        import pickle
+
+        from megakernels_amd.scheduler import assign_to_sms
+        from megakernels_amd.scripts.timeline import reference_event_layout
+
+        if config.start_after_op is None:
+            queues = assign_to_sms(config.sched, schedule=schedule)
+        else:
+            queues = assign_to_sms("rr", instructions=instructions, sm_count=config.workers)
+        gg = schedule_gpu.globs
+        outdata = {
+            "timings": reference_event_layout(gg.timings, gg.instructions),
+            "timings_native": gg.timings.cpu(),
+            "instructions": gg.instructions.cpu(),
+            "python_instructions": queues,
+            "cost_per_sm": [sum(ins.cost(g) for ins in q) for q in queues],
+        }
+        print(f"Saving to {config.outfile}")
+        with open(config.outfile, "wb") as f:
+            pickle.dump(outdata, f)
 
 
 if __name__ == "__main__":

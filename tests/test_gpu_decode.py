@@ -109,6 +109,47 @@ def test_decode_8b_slice_all_steps_in_one_launch():
     _decode_case(config_8b_slice(layers=2), workers=256, prefill=50, ntok=4, partitions=2, fused=True, steps_per_launch=0)
 
 
+def test_prefill_on_the_gpu_hands_its_cache_to_the_megakernel():
+    """The reference's flow (scripts/generate.py:125-137): the prompt goes through the plain PyTorch
+    forward on the GPU, which fills the KV cache and yields the first token; the megakernel decodes
+    from there.  The checker starts from a copy of the cache the GPU prefill left, and must see the
+    same tokens and the same appended KV rows."""
+    from megakernels_amd.generators import MK_Generator
+    from megakernels_amd.model_types import BatchState
+    from oracle import pyvm
+
+    cfg = config_1b_slice(layers=3)
+    model = make_model(cfg, max_len=128)
+    model_gpu = model.to("cuda:0")
+    prompt = torch.randint(0, cfg.vocab_size, (1, 32), generator=torch.Generator().manual_seed(1))
+    out = model_gpu(BatchState(input_ids=prompt.to("cuda:0"), position_ids=torch.arange(32, device="cuda:0")))
+    first_token = int(out.output_ids[0, -1])
+    for dst, src in zip(model.stacked_kv_cache, model_gpu.stacked_kv_cache):
+        dst.copy_(src)
+    assert float(model.stacked_kv_cache[0][:, :, :32].float().abs().sum()) > 0 and float(model.stacked_kv_cache[0][:, :, 32:].float().abs().sum()) == 0
+    # the GPU prefill agrees with the CPU forward to bf16 rounding (different GEMM kernels, same maths)
+    model_ref = make_model(cfg, max_len=128)
+    model_ref(BatchState(input_ids=prompt, position_ids=torch.arange(32)))
+    k_gpu, k_cpu = model.stacked_kv_cache[0][:, :, :32].float(), model_ref.stacked_kv_cache[0][:, :, :32].float()
+    assert float((k_gpu - k_cpu).abs().max()) <= 2e-2 * float(k_cpu.abs().max())
+
+    ntok = 8
+    schedule = build_schedule(model, 256)
+    _, schedule_gpu = mirror_to_gpu(model, schedule, model_gpu=model_gpu)
+    interp, mk_mod = _interpreter()
+    tokens_cpu = torch.zeros(1, ntok + 1, dtype=torch.long)
+    tokens_cpu[0, 0] = first_token
+    pyvm.OracleGenerator(model, schedule).generate(tokens_cpu, prompt_len=32, ntok=ntok)
+    tokens_gpu = torch.zeros(1, ntok + 1, dtype=torch.long, device="cuda:0")
+    tokens_gpu[0, 0] = first_token
+    MK_Generator(model_gpu, interp, schedule_gpu, fused_step=True, steps_per_launch=0).generate(
+        tokens_gpu, prompt_len=32, ntok=ntok, check=True)
+    assert tokens_gpu.cpu().tolist() == tokens_cpu.tolist()
+    names = [n for n in schedule.globs.mutable_tensor_names() if n != "barriers"]
+    report = mismatches(schedule.globs, schedule_gpu.globs, names=names, kv_rows=slice(0, 32 + ntok))
+    assert not report, report
+
+
 def test_decode_from_a_hugging_face_checkpoint(tmp_path):
     """The whole user path: a checkpoint directory written by the installed third-party `transformers`
     (untied head, llama3 rope scaling), loaded with `from_pretrained`, decoded through the megakernel,

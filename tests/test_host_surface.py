@@ -321,3 +321,27 @@ def test_repl_conversation_on_the_pytorch_generator(tmp_path):
     assert cfg.mode == "torch" and cfg.max_tokens_per_turn == 8 and cfg.print_prompt_len is True
     with pytest.raises(SystemExit):
         parse_args(["mode=mk"])
+
+
+def test_timing_records_in_the_reference_event_slots():
+    """scripts/timeline.reference_event_layout: the kernel's five stamps per instruction (low 32 bits
+    of one device clock) re-laid into the reference's event slots (include/util.cuh:215-246), as ticks
+    since the first instruction started - also across a wrap of the 32-bit clock."""
+    from megakernels_amd.scripts.timeline import REFERENCE_EVENTS, reference_event_layout
+
+    ins = torch.zeros(2, 3, 32, dtype=torch.int32)
+    ins[0, 0, 0], ins[0, 1, 0], ins[1, 0, 0] = 1, 6, 2          # worker 1 has two NoOps
+    raw = torch.zeros(2, 3, 128, dtype=torch.int64)
+    base = (1 << 32) - 50                                         # the clock wraps during the launch
+    raw[0, 0, :6] = torch.tensor([base + 0, base + 10, base + 20, base + 70, base + 90, 1])
+    raw[0, 1, :6] = torch.tensor([base + 100, base + 100, base + 130, base + 400, base + 420, 6])
+    raw[1, 0, :6] = torch.tensor([base + 5, base + 40, base + 45, base + 300, base + 310, 2])
+    timings = (raw & 0xFFFFFFFF).to(torch.int32)                 # what the kernel stores
+    out = reference_event_layout(timings, ins)
+    assert out.shape == timings.shape and out.dtype == torch.int32
+    assert out[0, 0, 0] == 0 and out[0, 0, 4] == 90 and out[0, 0, 45] == 10 and out[0, 0, 11] == 20 and out[0, 0, 46] == 70
+    assert out[0, 1, 0] == 100 and out[0, 1, 47] == 420 and out[1, 0, 0] == 5 and out[1, 0, 54] == 310
+    assert int(out[1, 1:].abs().sum()) == 0 and int(out[0, 2].abs().sum()) == 0
+    unused = [i for i in range(128) if i not in REFERENCE_EVENTS]
+    assert int(out[:, :, unused].abs().sum()) == 0
+    assert REFERENCE_EVENTS[0] == 0 and REFERENCE_EVENTS[4] == 4   # controller start / end coincide with the kernel's own

@@ -211,6 +211,11 @@ def test_split_kv_schedule():
     assert pick_num_attention_partitions(4096, 64) == 17
     assert pick_num_attention_partitions(32, 128) == 1
     assert pick_num_attention_partitions(16384, 64) == 24
+    set_sm_count_override(256)
+    assert pick_num_attention_partitions(16384, 64, num_kv_heads=8) == 32     # one per worker and KV head
+    assert pick_num_attention_partitions(4096, 64, num_kv_heads=8) == 17
+    set_sm_count_override(132)
+    assert pick_num_attention_partitions(16384, 64, num_kv_heads=8) == 24
 
 
 @pytest.mark.parametrize("P", [26, 32, 64])
