@@ -186,9 +186,6 @@ struct Smem {
     Consts k;
     mk_llama_args args;             // the launch arguments, read from here by every instruction
     int flags[16];                  // scratch of the end-of-step reduction
-#ifdef MK_TRACE_CONSUMER
-    int consumer_ticks[16];         // development trace: consumer timestamps parked until the instruction ends
-#endif
     alignas(16) uint32_t x[kMaxK / 2];          // activation vector as bf16 pairs, lane layout [chunk][lane][4 dwords]
     alignas(16) float out[kOutRows];            // matvec row results awaiting the epilogue
     alignas(16) float wave_max[kConsumerWaves][kGqa];
@@ -452,19 +449,6 @@ enum {
 
 __device__ __forceinline__ void trace_event(const Ctx &c, int slot) {
     if (c.trace && c.controller && c.lane == 0) st_plain_i32(c.trace + slot, (int)(uint32_t)wall_clock64());
-}
-
-// consumer-side events (wave 0, lane 0), slots 16 and up; for kernel development
-__device__ __forceinline__ void trace_consumer(const Ctx &c, int slot) {
-#ifdef MK_TRACE_CONSUMER
-    if (c.trace && c.tid == 0) c.sm->consumer_ticks[slot - 16] = (int)(uint32_t)wall_clock64();
-#endif
-}
-__device__ __forceinline__ void trace_consumer_flush(const Ctx &c, int first, int last) {
-#ifdef MK_TRACE_CONSUMER
-    if (c.trace && c.tid == 0)
-        for (int s = first; s <= last; s++) st_plain_i32(c.trace + s, c.sm->consumer_ticks[s - 16]);
-#endif
 }
 
 __device__ __forceinline__ int *bar_ptr(const Ctx &c, int layer, int row, int col) {
@@ -763,15 +747,11 @@ __device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need
         if (c.lane == 0) c.sm->out[c.wave + i * kConsumerWaves] = y;
     };
     wg_barrier();  // entry: the controller's first requests are out
-    trace_consumer(c, 20);
 #pragma unroll
     for (int s = 0; s < PF; s++) request(buf[s], s);
-    trace_consumer(c, 21);
     if (!barrier_inputs_ready(c, true)) return false;
-    trace_consumer(c, 22);
     XVec<KC> x;
     if (need_x) x_from_lds<KC>(x, c.sm, c.lane);
-    trace_consumer(c, 24);
     int base = 0;
     // rounds that are followed by more rows: every row of the round exists, every slot is refilled
     for (; base + PF < mine; base += PF) {
@@ -783,14 +763,11 @@ __device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need
             compiler_fence();
         }
     }
-    trace_consumer(c, 25);
     // last round: nothing left to request
 #pragma unroll
     for (int s = 0; s < PF; s++)
         if (base + s < mine) consume(buf[s], base + s, x);
-    trace_consumer(c, 23);
     wg_barrier();
-    trace_consumer_flush(c, 20, 25);
     // hold the next instruction's weight requests back until the controller has sent this
     // instruction's results and signal: they would otherwise queue behind the bulk loads
     wg_barrier();
@@ -1255,10 +1232,8 @@ __device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&pool)[NBUF][K
                                              MK_LDS const unsigned char *slice = nullptr) {
     constexpr int PF = Map::size;
     if (!barrier_inputs_ready(c, true)) return false;
-    trace_consumer(c, 22);
     XVec<KC> x;
     if (d.ntasks > 0) x_from_lds<KC>(x, c.sm, c.lane);
-    trace_consumer(c, 24);
     auto consume = [&](const uint4 (&src)[KC], int i) {
         const float y = mkm::round_bf16(dot_row<KC>(src, x));
         if (c.lane == 0) c.sm->out[c.wave + i * kConsumerWaves] = y;
@@ -1277,7 +1252,6 @@ __device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&pool)[NBUF][K
             compiler_fence();
         }
     }
-    trace_consumer(c, 25);
     // last round: nothing left to request
 #pragma unroll
     for (int s = 0; s < PF; s++)
@@ -1296,7 +1270,6 @@ __device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&pool)[NBUF][K
                 consume(row, parked_first + r);
             }
     }
-    trace_consumer(c, 23);
     wg_barrier();  // results are in LDS
     // hold further weight requests back until the controller has sent this instruction's results and
     // signal: they would otherwise queue behind the bulk loads
@@ -1338,11 +1311,8 @@ static __device__ __noinline__ bool op_matvec(SmemPtr lds, int slot, int *refusa
     const int mine = rows_of_wave(d.ntasks, c.wave);
     uint4 pool[PF][KC];
     wg_barrier();  // entry: the controller's first requests are out
-    trace_consumer(c, 20);
     request_rows<KC, Map>(c, pool, d, 0, mine > PARKED ? mine - PARKED : 0);
-    trace_consumer(c, 21);
     const bool ok = consumer_run<KC, Map, PF, PARKED>(c, pool, d, mine, (MK_LDS const unsigned char *)lds->park + c.wave * (KC * 1024));
-    trace_consumer_flush(c, 20, 25);
     return ok;
 }
 
@@ -1651,7 +1621,6 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
         }
     }
     if (!barrier_inputs_ready(c, true)) return false;
-    trace_consumer(c, 16);
 
     float q[G][8];
     {
@@ -1670,7 +1639,6 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
 #pragma unroll
         for (int h = 0; h < G; h++) unpack8(qraw[h], q[h]);
     }
-    trace_consumer(c, 17);
 
     // scores of one token against the four heads, valid in all lanes of the token's group
     auto scores_of = [&](const uint4 &krow, float (&sc)[G]) {
@@ -1717,16 +1685,13 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
             if (r < T) score_round(kb[u], r);
         }
     }
-    trace_consumer(c, 18);
     {
         float m[G];
 #pragma unroll
         for (int h = 0; h < G; h++) m[h] = lane_tree_max<LPT, 64>(mx[h]);
         if (c.lane == 0) *(MK_LDS f32x4 *)&sm->wave_max[c.wave][0] = f32x4{m[0], m[1], m[2], m[3]};
     }
-    trace_consumer(c, 19);
     wg_barrier();
-    trace_consumer_flush(c, 16, 19);
     float hm[G];
     {
         f32x4 m = *(const MK_LDS f32x4 *)&sm->wave_max[0][0];
@@ -1851,7 +1816,6 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
     // ---- combine the 8 waves pairwise, normalise, store: thread -> (head, dim pair).  The threads of
     // one head sit in one wave, which signals for that head once its own stores have landed. ----
     if (c.tid < G * D / 2) {
-        trace_consumer(c, 29);
         const int h = c.tid / (D / 2), d = (c.tid % (D / 2)) * 2;
         float o0[kConsumerWaves], o1[kConsumerWaves], l[kConsumerWaves];
 #pragma unroll
@@ -1887,14 +1851,11 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
             st_f32(dst + 1, r1);
             if (d == 0) st_f32(a.attn_lse_intermediates + (size_t)head * a.max_partials + pidx, lse);
         }
-        trace_consumer(c, 30);
         wait_stores();
-        trace_consumer(c, 31);
         if (d == 0) {
             if (skip) signal_sharded_lane(c, layer, 2, 1);
             else add_i32(pad_ptr(c, layer, 1, head), 1);
         }
-        trace_consumer_flush(c, 29, 31);
     }
     return true;
 }
@@ -1933,9 +1894,7 @@ static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot
         const PollTicket ticket =
             poll_issue(c, leader ? pad_ptr(c, layer, 1, head) : nullptr, leader ? bar_ptr(c, layer, 1, head) : nullptr);
         if (poll_wait(c, ticket, false, P, []() {})) {
-            trace_consumer(c, 26);
             const MergedPair r = merge_partitions<D>(c, head, j, n, [&](int k) { return ins[6 + k]; });
-            trace_consumer(c, 27);
             if (terminal) {
                 st_u32(a.attn_out + (size_t)head * D + d, mkm::pack_bf16(r.o0, r.o1));
             } else {
@@ -1952,8 +1911,6 @@ static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot
                 if (terminal) signal_sharded_lane(c, layer, 2, 1);
                 else add_i32(pad_ptr(c, layer, 1, head), 1);
             }
-            trace_consumer(c, 28);
-            trace_consumer_flush(c, 26, 28);
         } else if (c.lane == 0) {
             c.sm->abort = 1;
         }
