@@ -174,6 +174,14 @@ int mk_llama_query(int what);
  * test suites, not for the decode path.  Must report 0. */
 int mk_llama_selftest_bf16(uint64_t *mismatches_out);
 
+/* Self test (no counterpart in the reference): out[i] = acc[i] + a[i].lo * b[i].lo + a[i].hi * b[i].hi
+ * computed by the instruction the kernel's matvec dot products are built from (V_DOT2_F32_BF16;
+ * a, b: 32-bit words holding two bf16, lo = bits 0-15; acc, out: binary32), over n <= 2^31 cases in
+ * device memory, asynchronously on `hip_stream`.  The instruction's arithmetic is not a chain of
+ * IEEE operations; test suites compare its results with the written-out definition they check the
+ * kernel against.  Allocates nothing. */
+int mk_llama_selftest_dot2(const void *a, const void *b, const void *acc, void *out, uint64_t n, void *hip_stream);
+
 const char *mk_llama_last_error(void);
 
 #ifdef __cplusplus

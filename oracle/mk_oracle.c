@@ -27,11 +27,15 @@
  *   attention     fp32 throughout; bf16 only when written to attn_out              (:316-330)
  *
  * Canonical summation order ("column order"):
- *   dot product over K elements (K a multiple of 512): 512 column accumulators;
- *   column c accumulates elements j*512 + c (j = 0..K/512-1) in order of j with
- *   fused multiply-add starting from 0; the 512 column sums are then added
- *   pairwise as a balanced binary tree in column-index order ((0+1)+(2+3))+... .
- *   The sum of squares of the RMS norm is formed the same way.
+ *   matvec dot product over K elements (K a multiple of 512), both operands bf16:
+ *   256 accumulators; accumulator c takes the element pairs j*256 + c (elements
+ *   2(j*256 + c) and the next; j = 0..K/512-1) in order of j, each step being the
+ *   two-element dot product acc + w0*x0 + w1*x1 of exact_math.h (orc_dot2_bf16:
+ *   the arithmetic of the GPU's instruction for it, not a chain of IEEE
+ *   operations), starting from 0; the 256 sums are then added (IEEE fp32)
+ *   pairwise as a balanced binary tree in index order ((0+1)+(2+3))+... .
+ *   The sum of squares of the RMS norm: 512 column accumulators, column c
+ *   accumulates elements j*512 + c in order of j with fused multiply-add, same tree.
  *   A head-dimension dot product uses D/8 lanes; lane l accumulates its elements
  *   l*8 .. l*8+7 in order with fused multiply-add and the lanes are added as a
  *   balanced binary tree.
@@ -94,13 +98,19 @@ static float tree_sum(float *v, int n) { /* n a power of two; destroys v */
     return v[0];
 }
 
-/* dot(w[0..K), x[0..K)), w bf16, x fp32, column order */
+/* dot(w[0..K), x[0..K)), w bf16, x fp32 holding bf16 values (every matvec input of the VM is a
+ * bf16 tensor), column order */
 static float dot_lanes(const uint16_t *w, const float *x, int K) {
-    float acc[512];
-    for (int c = 0; c < 512; c++) acc[c] = 0.0f;
+    float acc[256];
+    for (int c = 0; c < 256; c++) acc[c] = 0.0f;
     for (int j = 0; j < K; j += 512)
-        for (int c = 0; c < 512; c++) acc[c] = fmaf(orc_bf16_to_f32(w[j + c]), x[j + c], acc[c]);
-    return tree_sum(acc, 512);
+        for (int c = 0; c < 256; c++) {
+            const int i = j + 2 * c;
+            const uint32_t wp = (uint32_t)w[i] | ((uint32_t)w[i + 1] << 16);
+            const uint32_t xp = (orc_f32_bits(x[i]) >> 16) | (orc_f32_bits(x[i + 1]) & 0xffff0000u);
+            acc[c] = orc_dot2_bf16(wp, xp, acc[c]);
+        }
+    return tree_sum(acc, 256);
 }
 
 /* python_vm.py:50-56.  out[i] = float(bf16(w[i] * bf16(x[i] * rsqrt(mean(x^2) + eps)))) */
@@ -469,3 +479,7 @@ float mk_oracle_exp2f(float x) { return orc_exp2f(x); }
 float mk_oracle_log2f(float x) { return orc_log2f(x); }
 uint16_t mk_oracle_f32_to_bf16(float x) { return orc_f32_to_bf16(x); }
 float mk_oracle_dot(const uint16_t *w, const float *x, int K) { return dot_lanes(w, x, K); }
+void mk_oracle_dot2(const uint32_t *a, const uint32_t *b, const float *acc, float *out, size_t n) {
+#pragma omp parallel for
+    for (size_t i = 0; i < n; i++) out[i] = orc_dot2_bf16(a[i], b[i], acc[i]);
+}

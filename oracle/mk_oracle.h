@@ -58,5 +58,8 @@ float mk_oracle_exp2f(float x);
 float mk_oracle_log2f(float x);
 uint16_t mk_oracle_f32_to_bf16(float x);
 float mk_oracle_dot(const uint16_t *w, const float *x, int K);
+/* out[i] = acc[i] + a[i].lo * b[i].lo + a[i].hi * b[i].hi (bf16 pairs), the two-element dot product
+ * of exact_math.h */
+void mk_oracle_dot2(const uint32_t *a, const uint32_t *b, const float *acc, float *out, size_t n);
 
 #endif

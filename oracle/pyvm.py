@@ -75,8 +75,22 @@ def load_lib():
         lib.mk_oracle_f32_to_bf16.restype = ctypes.c_uint16
         lib.mk_oracle_dot.argtypes = [_U16P, _F32P, ctypes.c_int]
         lib.mk_oracle_dot.restype = ctypes.c_float
+        lib.mk_oracle_dot2.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]
+        lib.mk_oracle_dot2.restype = None
         _lib = lib
     return _lib
+
+
+def dot2(a, b, acc):
+    """acc + a.lo * b.lo + a.hi * b.hi per element: numpy uint32 bf16 pairs and float32 accumulators."""
+    import numpy as np
+
+    a = np.ascontiguousarray(a, dtype=np.uint32)
+    b = np.ascontiguousarray(b, dtype=np.uint32)
+    acc = np.ascontiguousarray(acc, dtype=np.float32)
+    out = np.empty_like(acc)
+    load_lib().mk_oracle_dot2(a.ctypes.data, b.ctypes.data, acc.ctypes.data, out.ctypes.data, a.size)
+    return out
 
 
 class OracleError(AssertionError):

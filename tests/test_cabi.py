@@ -31,7 +31,8 @@ def load():
 
 def test_header_declares_the_expected_entry_points():
     assert declared_functions() == ["mk_llama_last_error", "mk_llama_launch", "mk_llama_launch_static", "mk_llama_query",
-                                    "mk_llama_read_status", "mk_llama_selftest_bf16", "mk_llama_workspace_bytes"]
+                                    "mk_llama_read_status", "mk_llama_selftest_bf16", "mk_llama_selftest_dot2",
+                                    "mk_llama_workspace_bytes"]
 
 
 def test_library_exports_every_declared_symbol():
