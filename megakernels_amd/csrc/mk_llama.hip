@@ -1636,11 +1636,10 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
     }
     if (!barrier_inputs_ready(c, true)) return false;
 
-    float q[G][8];
+    uint4 q[G];  // this lane's 8 dims of the four query heads, as bf16 pairs
     {
-        uint4 qraw[G];
 #pragma unroll
-        for (int h = 0; h < G; h++) qraw[h] = ld_b128(a.q_post_rope + (size_t)(h0 + h) * D + sub * 8);
+        for (int h = 0; h < G; h++) q[h] = ld_b128(a.q_post_rope + (size_t)(h0 + h) * D + sub * 8);
         // the newest token's rows, if they fall into the first batch
 #pragma unroll
         for (int u = 0; u < RU; u++) {
@@ -1650,19 +1649,16 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
                 vraw[u] = ld_b128(vbase + (size_t)(t0 + r) * tok_stride);
             }
         }
-#pragma unroll
-        for (int h = 0; h < G; h++) unpack8(qraw[h], q[h]);
     }
 
     // scores of one token against the four heads, valid in all lanes of the token's group
     auto scores_of = [&](const uint4 &krow, float (&sc)[G]) {
-        float kf[8];
-        unpack8(krow, kf);
 #pragma unroll
         for (int h = 0; h < G; h++) {
-            float acc = 0.0f;
-#pragma unroll
-            for (int e = 0; e < 8; e++) acc = fmaf(q[h][e], kf[e], acc);
+            float acc = dot2_bf16(krow.x, q[h].x, 0.0f);
+            acc = dot2_bf16(krow.y, q[h].y, acc);
+            acc = dot2_bf16(krow.z, q[h].z, acc);
+            acc = dot2_bf16(krow.w, q[h].w, acc);
             sc[h] = group_tree_sum<LPT>(acc) * a.attn_scale;
         }
     };

@@ -36,9 +36,9 @@
  *   pairwise as a balanced binary tree in index order ((0+1)+(2+3))+... .
  *   The sum of squares of the RMS norm: 512 column accumulators, column c
  *   accumulates elements j*512 + c in order of j with fused multiply-add, same tree.
- *   A head-dimension dot product uses D/8 lanes; lane l accumulates its elements
- *   l*8 .. l*8+7 in order with fused multiply-add and the lanes are added as a
- *   balanced binary tree.
+ *   A head-dimension dot product (query . key, both bf16) uses D/8 lanes; lane l
+ *   accumulates its element pairs (l*8, l*8+1) .. (l*8+6, l*8+7) in order with the
+ *   two-element dot product and the lanes are added as a balanced binary tree.
  *   Attention over a token range: relative token r goes to slot r mod NSLOT
  *   (NSLOT = 4096/D); each slot accumulates its tokens in increasing order
  *   (fused multiply-add for p*v, plain add for the denominator); the slots
@@ -240,7 +240,6 @@ static int op_partial_attention(mk_oracle_globals *g, const int32_t *w) {
         float *scores = (float *)malloc(sizeof(float) * (T > 0 ? T : 1));
         float *lslot = (float *)malloc(sizeof(float) * NSLOT);
         float *oslot = (float *)malloc(sizeof(float) * NSLOT * D);
-        float *q = (float *)malloc(sizeof(float) * D);
         float *col = (float *)malloc(sizeof(float) * NSLOT);
         float out[256];
         float lse;
@@ -248,14 +247,16 @@ static int op_partial_attention(mk_oracle_globals *g, const int32_t *w) {
             for (int d = 0; d < D; d++) out[d] = 0.0f;
             lse = -INFINITY;
         } else {
-            for (int d = 0; d < D; d++) q[d] = orc_bf16_to_f32(g->post_ln_rope_q[head * D + d]);
+            const uint16_t *qb = g->post_ln_rope_q + head * D;
             float m = -INFINITY;
             for (int r = 0; r < T; r++) {
                 const uint16_t *k = kbase + (size_t)(t0 + r) * tok_stride;
                 float lane[16];
                 for (int i = 0; i < LPT; i++) {
                     float a = 0.0f;
-                    for (int e = 0; e < 8; e++) a = fmaf(q[i * 8 + e], orc_bf16_to_f32(k[i * 8 + e]), a);
+                    for (int e = 0; e < 8; e += 2)
+                        a = orc_dot2_bf16((uint32_t)k[i * 8 + e] | ((uint32_t)k[i * 8 + e + 1] << 16),
+                                          (uint32_t)qb[i * 8 + e] | ((uint32_t)qb[i * 8 + e + 1] << 16), a);
                     lane[i] = a;
                 }
                 float s = tree_sum(lane, LPT) * g->attn_scale;
@@ -286,7 +287,7 @@ static int op_partial_attention(mk_oracle_globals *g, const int32_t *w) {
             memcpy(g->attn_out_intermediates + ((size_t)head * g->max_partials + pidx) * D, out,
                    sizeof(float) * D);
         }
-        free(scores); free(lslot); free(oslot); free(q); free(col);
+        free(scores); free(lslot); free(oslot); free(col);
     }
 
     if (g->skip_attn_reduction) BAR(g, layer, 2, 0) += G;
