@@ -484,3 +484,7 @@ void mk_oracle_dot2(const uint32_t *a, const uint32_t *b, const float *acc, floa
 #pragma omp parallel for
     for (size_t i = 0; i < n; i++) out[i] = orc_dot2_bf16(a[i], b[i], acc[i]);
 }
+void mk_oracle_dot2_general(const uint32_t *a, const uint32_t *b, const float *acc, float *out, size_t n) {
+#pragma omp parallel for
+    for (size_t i = 0; i < n; i++) out[i] = orc_dot2_bf16_general(a[i], b[i], acc[i]);
+}

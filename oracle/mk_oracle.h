@@ -61,5 +61,7 @@ float mk_oracle_dot(const uint16_t *w, const float *x, int K);
 /* out[i] = acc[i] + a[i].lo * b[i].lo + a[i].hi * b[i].hi (bf16 pairs), the two-element dot product
  * of exact_math.h */
 void mk_oracle_dot2(const uint32_t *a, const uint32_t *b, const float *acc, float *out, size_t n);
+/* the same through the clause-by-clause form only (orc_dot2_bf16 takes a shorter way for ordinary operands) */
+void mk_oracle_dot2_general(const uint32_t *a, const uint32_t *b, const float *acc, float *out, size_t n);
 
 #endif

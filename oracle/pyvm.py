@@ -77,19 +77,23 @@ def load_lib():
         lib.mk_oracle_dot.restype = ctypes.c_float
         lib.mk_oracle_dot2.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]
         lib.mk_oracle_dot2.restype = None
+        lib.mk_oracle_dot2_general.argtypes = lib.mk_oracle_dot2.argtypes
+        lib.mk_oracle_dot2_general.restype = None
         _lib = lib
     return _lib
 
 
-def dot2(a, b, acc):
-    """acc + a.lo * b.lo + a.hi * b.hi per element: numpy uint32 bf16 pairs and float32 accumulators."""
+def dot2(a, b, acc, general: bool = False):
+    """acc + a.lo * b.lo + a.hi * b.hi per element: numpy uint32 bf16 pairs and float32 accumulators.
+    ``general``: through the clause-by-clause form only."""
     import numpy as np
 
     a = np.ascontiguousarray(a, dtype=np.uint32)
     b = np.ascontiguousarray(b, dtype=np.uint32)
     acc = np.ascontiguousarray(acc, dtype=np.float32)
     out = np.empty_like(acc)
-    load_lib().mk_oracle_dot2(a.ctypes.data, b.ctypes.data, acc.ctypes.data, out.ctypes.data, a.size)
+    fn = load_lib().mk_oracle_dot2_general if general else load_lib().mk_oracle_dot2
+    fn(a.ctypes.data, b.ctypes.data, acc.ctypes.data, out.ctypes.data, a.size)
     return out
 
 

@@ -156,6 +156,14 @@ def test_dot2_definition_against_the_instructions_results():
     got = pyvm.dot2(a, b, acc.view(np.float32)).view(np.uint32)
     bad = np.flatnonzero(~dot2_cases.same_results(got, out))
     assert bad.size == 0, [(hex(a[i]), hex(b[i]), hex(acc[i]), hex(out[i]), hex(got[i])) for i in bad[:5]]
+    # the clause-by-clause form alone, and both forms on fresh operands of every class
+    assert dot2_cases.same_results(pyvm.dot2(a, b, acc.view(np.float32), general=True).view(np.uint32), out).all()
+    rng = np.random.default_rng(99)
+    for gen in dot2_cases.CLASSES:
+        x, y, z = (np.ascontiguousarray(t, dtype=np.uint32) for t in gen(rng, 200000))
+        short = pyvm.dot2(x, y, z.view(np.float32)).view(np.uint32)
+        full = pyvm.dot2(x, y, z.view(np.float32), general=True).view(np.uint32)
+        assert dot2_cases.same_results(short, full).all(), gen.__name__
     # every class is present and none is trivial: results differ from a fused multiply-add chain somewhere
     per = int(v["per_class"])
     assert len(a) == per * len(v["classes"]) and list(v["classes"]) == [g.__name__ for g in dot2_cases.CLASSES]
