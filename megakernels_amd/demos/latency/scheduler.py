@@ -61,16 +61,21 @@ from megakernels_amd.utils import assert_div, get_sm_count
 MAX_ATTENTION_PARTITIONS = INTS_PER_INSTRUCTION - 7
 
 
-def pick_num_attention_partitions(prompt_len: int, ntok: int, device=None, num_kv_heads: int | None = None) -> int:
-    """One partition per 256 cached positions, at most 24 (reference ``:21-35``) - or, when the number
-    of KV heads is given, at most one partition per worker for every KV head if that is more (256
-    workers, 8 KV heads: 32): beyond 25 partitions the merges go through a reduction tree, which costs
-    a few microseconds per layer and pays once the partitions are long (16384 positions and up)."""
+def pick_num_attention_partitions(prompt_len: int, ntok: int, device=None, num_kv_heads: int | None = None,
+                                  head_dim: int | None = None) -> int:
+    """One partition per 256 cached positions, at most 24 (reference ``:21-35``) - or, when the shape of the
+    KV heads is given, up to one partition per worker for every KV head (256 workers, 8 KV heads: 32).
+    Beyond 25 partitions the merges go through a reduction tree, which costs a few microseconds per layer
+    and pays once a partition job would otherwise stream more than 384 KB of K and V rows (8B shapes from
+    about 20000 positions; the 1B shape at 16384 positions is faster with 24)."""
     min_chunk_size = 256
-    num_divisions = math.ceil((prompt_len + ntok) / min_chunk_size)
+    length = prompt_len + ntok
+    num_divisions = math.ceil(length / min_chunk_size)
     most = 24
-    if num_kv_heads:
-        most = max(most, get_sm_count(device if device is not None else "cuda") // num_kv_heads)
+    if num_kv_heads and head_dim:
+        job_bytes = math.ceil(length / most) * head_dim * 2 * 2
+        if job_bytes > 384 * 1024:
+            most = max(most, get_sm_count(device if device is not None else "cuda") // num_kv_heads)
     return max(1, min(num_divisions, most))
 
 

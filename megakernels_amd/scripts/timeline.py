@@ -112,7 +112,7 @@ def main(argv):
     model = model.to(device)
     workers = get_sm_count(device)
     set_sm_count_override(workers)
-    partitions = opts["partitions"] or pick_num_attention_partitions(pos, 1, device, cfg.num_key_value_heads)
+    partitions = opts["partitions"] or pick_num_attention_partitions(pos, 1, device, cfg.num_key_value_heads, cfg.head_dim)
     schedule = LatencyScheduleBuilder.build(model, num_attention_partitions=partitions)
     tensorize_instructions(schedule.globs, assign_to_sms(opts["sched"], schedule=schedule))
     globs = schedule.globs

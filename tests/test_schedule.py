@@ -212,10 +212,12 @@ def test_split_kv_schedule():
     assert pick_num_attention_partitions(32, 128) == 1
     assert pick_num_attention_partitions(16384, 64) == 24
     set_sm_count_override(256)
-    assert pick_num_attention_partitions(16384, 64, num_kv_heads=8) == 32     # one per worker and KV head
-    assert pick_num_attention_partitions(4096, 64, num_kv_heads=8) == 17
-    set_sm_count_override(132)
+    assert pick_num_attention_partitions(32768, 64, num_kv_heads=8, head_dim=128) == 32   # one per worker and KV head
+    assert pick_num_attention_partitions(16384, 64, num_kv_heads=8, head_dim=64) == 24    # jobs too short for a tree
     assert pick_num_attention_partitions(16384, 64, num_kv_heads=8) == 24
+    assert pick_num_attention_partitions(4096, 64, num_kv_heads=8, head_dim=64) == 17
+    set_sm_count_override(132)
+    assert pick_num_attention_partitions(32768, 64, num_kv_heads=8, head_dim=128) == 24
 
 
 @pytest.mark.parametrize("P", [26, 32, 64])
