@@ -80,6 +80,7 @@ def main():
                     help="decode steps also timed on the torch restatement of the Python VM, the closer stand-in for "
                          "the reference's python_vm.py (0 = skip; default 3 for 1B, 1 for 8B)")
     ap.add_argument("--sched", default="rr")
+    ap.add_argument("--workers", type=int, default=0, help="instruction queues (0 = one per compute unit)")
     ap.add_argument("--partitions", type=int, default=0, help="attention partitions (0 = one per 256 positions, at most 24, or one per worker and KV head when the jobs are long)")
     ap.add_argument("--loop", default="fused", choices=["fused", "reference"],
                     help="fused: one launch per token (embedding row, barrier reset and argmax inside the "
@@ -151,7 +152,7 @@ def main():
         for dst, src in zip(model_cpu.stacked_kv_cache, model.stacked_kv_cache):
             dst.copy_(src)
 
-    workers = get_sm_count(device)
+    workers = args.workers or get_sm_count(device)
     set_sm_count_override(workers)
     partitions = args.partitions or pick_num_attention_partitions(prefill, total_steps, device, cfg.num_key_value_heads, cfg.head_dim)
 
