@@ -121,3 +121,10 @@ def test_c5_full_8b_32768_positions_24_partitions(full_8b):
     schedule, _ = _one_step(full_8b, pos=32770, partitions=24)
     assert schedule.globs.instructions.shape[1] >= 150
     _decode(full_8b, prefill=32770, ntok=3, partitions=24)
+
+
+def test_c5_full_8b_32768_positions_32_partitions_through_the_tree(full_8b):
+    """the partition count the benchmark picks for this shape: one job per worker and KV head, merged by a
+    two-level reduction tree; every partition streams 1024 positions through the double-buffered row stream"""
+    _one_step(full_8b, pos=32770, partitions=32)
+    _decode(full_8b, prefill=32770, ntok=2, partitions=32)
