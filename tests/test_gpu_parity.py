@@ -158,6 +158,21 @@ def test_single_partition_beyond_the_score_buffer():
     _one_step_case(_tiny_long_context(16448), workers=16, pos=16384, max_len=16384 + 64)
 
 
+@pytest.mark.parametrize("pos", [255, 256, 257, 319, 511, 512, 513, 767, 768, 1023, 1024, 1025, 1300])
+def test_tiny_row_stream_boundaries(pos):
+    """Partitions around the edges of the double-buffered row stream (head_dim 64: the first 256 positions
+    of a partition are requested ahead of the dependency, the rest streams in batches of 256): the newest
+    position first, last or alone in a batch, a batch that ends with the partition, one position beyond."""
+    _one_step_case(_tiny_long_context(2048), workers=16, pos=pos, max_len=1408)
+    _one_step_case(_tiny_long_context(2048), workers=16, pos=pos, partitions=2, max_len=1408)
+
+
+def test_8b_slice_row_stream_boundaries():
+    # head_dim 128: 128 positions ahead of the dependency, batches of 128
+    for pos in (127, 128, 129, 255, 256, 257, 400):
+        _one_step_case(config_8b_slice(), workers=256, pos=pos, partitions=1, max_len=512)
+
+
 def test_1b_slice_single_partition_long_context():
     _one_step_case(config_1b_slice(layers=1), workers=256, pos=5000, partitions=1, max_len=5120)
 
