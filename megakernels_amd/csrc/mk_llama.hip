@@ -39,11 +39,12 @@
 //     the others wait for that and start over one position further on.
 //
 // Arithmetic: bit-compatible with a fixed "column order" so results can be compared exactly
-// with a CPU restatement of the Python VM.  A dot product over K elements is computed by one
-// wave: column c = lane * 8 + e accumulates elements j*512 + c in order of j with fmaf (eight
-// independent chains per lane), the 512 column sums are combined as a balanced pairwise tree
-// (within the lane, then an xor butterfly over lanes).  Narrowing to bf16 happens exactly where
-// the Python VM narrows (python_vm.py:29-80,127-274).
+// with a CPU restatement of the Python VM.  A matvec dot product over K elements is computed by
+// one wave: accumulator c = lane * 4 + d takes the element pairs j*256 + c in order of j, each
+// step being the two-element bf16 dot product instruction (four independent chains per lane; its
+// arithmetic is written out where the test suite keeps its definition), and the 256 sums are
+// combined as a balanced pairwise tree (within the lane, then an xor butterfly over lanes).
+// Narrowing to bf16 happens exactly where the Python VM narrows (python_vm.py:29-80,127-274).
 #include <hip/hip_runtime.h>
 
 #include <climits>
