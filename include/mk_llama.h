@@ -22,7 +22,7 @@
 extern "C" {
 #endif
 
-#define MK_LLAMA_ABI_VERSION 5
+#define MK_LLAMA_ABI_VERSION 6
 #define MK_INSTRUCTION_WORDS 32   /* megakernels/scheduler.py:13, include/config.cuh:14 */
 #define MK_TIMING_SLOTS 128       /* megakernels/scheduler.py:14, include/config.cuh:18 */
 #define MK_BARRIER_ROWS 10        /* megakernels/demos/latency/scheduler.py:53-61 */
@@ -38,6 +38,18 @@ extern "C" {
  * the next launch needs no reset (the reference's loop refills the tensor before every launch,
  * megakernels/generators.py:127-128). */
 #define MK_FLAG_RESET_BARRIERS 2u
+/* args.flags: the caller promises that the residual projections' column-group jobs (opcodes 4 and 6
+ * with hidden_size or intermediate_size a multiple of matvec_reduction_size) come in complete sets:
+ * for every (opcode, layer, row block) that appears in `instructions`, the jobs of all column groups
+ * appear, each exactly once.  The jobs of a set then share their work by rows instead of by columns
+ * (the job of group c computes 16 / G of the block's rows over all G groups' columns and applies
+ * every group's sum to the residual itself, in group order), so no partial sums travel between
+ * workers and no job waits for another.  Results and barrier counts are those of executing each
+ * instruction on its own, which is what happens without the flag; with the flag set on an incomplete
+ * set, rows of hidden_states miss their update.  Every schedule of
+ * megakernels/demos/latency/scheduler.py:167-213,346-352 qualifies.  Used when the group count
+ * divides 8; other shapes run each job on its own regardless. */
+#define MK_FLAG_JOINT_RESIDUAL 4u
 
 /* Words of one instruction's timing record.  Words 0 and 4 are the reference's
  * TEVENT_CONTROLLER_START and TEVENT_CONTROLLER_END (include/util.cuh:215-219).  Words 1-3 are

@@ -59,8 +59,14 @@
 
 namespace {
 
-constexpr int kConsumerWaves = 8;
+#ifndef MK_CONSUMER_WAVES
+#define MK_CONSUMER_WAVES 8
+#endif
+constexpr int kConsumerWaves = MK_CONSUMER_WAVES;  // waves that stream weight rows in the matvec instructions
+constexpr int kAttnWaves = 8;       // waves that work on an attention partition (the token -> slot mapping is built on 8)
+static_assert(kConsumerWaves >= kAttnWaves, "attention runs on the first consumer waves");
 constexpr int kConsumerThreads = kConsumerWaves * 64;
+constexpr int kAttnThreads = kAttnWaves * 64;
 constexpr int kThreads = kConsumerThreads + 64;  // + one controller wave
 #ifndef MK_SHARDS
 #define MK_SHARDS 16
@@ -75,7 +81,6 @@ constexpr int kOutRows = 2048;      // rows staged in LDS between matvec and epi
 constexpr int kMaxK = 4096;         // longest activation vector handed through LDS
 constexpr int kScoreCap = 4096;     // tokens per attention partition (LDS score buffer)
 constexpr int kQueueSlots = 192;    // instructions of a worker's queue kept in LDS at a time (a longer queue goes through in windows)
-constexpr int kParkBytes = kConsumerWaves * 4096;  // one more parked row per wave, outside the score buffer
 constexpr int kMaxHeadDim = 128;
 constexpr int kGqa = 4;             // query heads per KV head handled by one attention instruction
 constexpr int kStatusInts = 16;
@@ -123,6 +128,7 @@ constexpr int rows_in_flight(int wanted) { return KC <= 4 ? wanted : (wanted < M
 #ifndef MK_POLL_SLEEP
 #define MK_POLL_SLEEP 10            // units of 64 clocks between two looks at a dependency
 #endif
+constexpr int kParkBytes = MK_PARK_DOWN ? kConsumerWaves * 4096 : 16;  // one more parked row per wave, outside the score buffer
 #define AG __HIP_MEMORY_SCOPE_AGENT
 
 // ---------------------------------------------------------------------------------------------
@@ -173,7 +179,8 @@ struct Consts {
 // ntasks < 0: the instruction is malformed.
 struct alignas(16) SlotDesc {
     uint64_t w0_base;               // buffer the rows are addressed in
-    long long gate_delta;           // opcode 5: byte distance from the up matrix to the gate matrix
+    long long gate_delta;           // opcode 5: byte distance from the up matrix to the gate matrix;
+                                    // opcodes 4, 6: column groups executed jointly (0: own group only)
     uint32_t w0_bytes, row_bytes;
     int ntasks, first_row;
 };
@@ -189,9 +196,9 @@ struct Smem {
     int flags[16];                  // scratch of the end-of-step reduction
     alignas(16) uint32_t x[kMaxK / 2];          // activation vector as bf16 pairs, lane layout [chunk][lane][4 dwords]
     alignas(16) float out[kOutRows];            // matvec row results awaiting the epilogue
-    alignas(16) float wave_max[kConsumerWaves][kGqa];
-    alignas(16) float wave_l[kConsumerWaves][kGqa];
-    alignas(16) float wave_o[kConsumerWaves][kGqa][kMaxHeadDim];
+    alignas(16) float wave_max[kAttnWaves][kGqa];
+    alignas(16) float wave_l[kAttnWaves][kGqa];
+    alignas(16) float wave_o[kAttnWaves][kGqa][kMaxHeadDim];
     alignas(16) float scores[kScoreCap][kGqa];  // attention: one partition's scores, then probabilities
     alignas(16) unsigned char park[kParkBytes];  // a weight row per wave parked for a later instruction
     int parked_slot;                               // the instruction whose last row per wave lies in `park`, or -1
@@ -623,10 +630,14 @@ __device__ __forceinline__ void load_xq(uint4 (&xq)[KC], const uint16_t *src, in
 // controller -> consumers hand-over of the activation vector: each lane's 16 bytes of a chunk are
 // adjacent to its neighbours', so the 128-bit LDS accesses are free of bank conflicts
 template <int KC>
-__device__ __forceinline__ void x_to_lds(const uint4 (&xq)[KC], SmemPtr sm, int lane) {
+__device__ __forceinline__ void x_to_lds(const uint4 (&xq)[KC], MK_LDS uint32_t *dst, int lane) {
 #pragma unroll
     for (int j = 0; j < KC; j++)
-        *(MK_LDS u32x4 *)(sm->x + (j * 64 + lane) * 4) = u32x4{xq[j].x, xq[j].y, xq[j].z, xq[j].w};
+        *(MK_LDS u32x4 *)(dst + (j * 64 + lane) * 4) = u32x4{xq[j].x, xq[j].y, xq[j].z, xq[j].w};
+}
+template <int KC>
+__device__ __forceinline__ void x_to_lds(const uint4 (&xq)[KC], SmemPtr sm, int lane) {
+    x_to_lds<KC>(xq, (MK_LDS uint32_t *)sm->x, lane);
 }
 // the consumers keep the vector as it lies in LDS: bf16 pairs, 4 dwords per lane and chunk
 template <int KC>
@@ -634,12 +645,16 @@ struct XPairs {
     uint4 v[KC];
 };
 template <int KC>
-__device__ __forceinline__ void x_from_lds(XPairs<KC> &x, SmemPtr sm, int lane) {
+__device__ __forceinline__ void x_from_lds(XPairs<KC> &x, const MK_LDS uint32_t *src, int lane) {
 #pragma unroll
     for (int j = 0; j < KC; j++) {
-        const u32x4 r = *(const MK_LDS u32x4 *)(sm->x + (j * 64 + lane) * 4);
+        const u32x4 r = *(const MK_LDS u32x4 *)(src + (j * 64 + lane) * 4);
         x.v[j] = uint4{r.x, r.y, r.z, r.w};
     }
+}
+template <int KC>
+__device__ __forceinline__ void x_from_lds(XPairs<KC> &x, SmemPtr sm, int lane) {
+    x_from_lds<KC>(x, (const MK_LDS uint32_t *)sm->x, lane);
 }
 
 // A weight row of an instruction: a buffer resource (uniform) and the row's byte offset in it.
@@ -816,6 +831,20 @@ struct MatvecDesc {
     InsPtr ins;
 };
 
+// Joint execution of a residual projection's column-group jobs (MK_FLAG_JOINT_RESIDUAL: the caller
+// promises that for every row block either all G column groups' jobs are in the instruction tensor
+// or none).  The G jobs of a block then share the work by rows instead of by columns: the job of
+// group c computes rows [c * 16 / G, (c + 1) * 16 / G) of the block over all G column groups, so it
+// holds every group's partial sum of its rows and applies them to the residual itself, in group order
+// - no partial sums travel between workers and no job waits for another.  Results and barrier counts
+// are those of the instruction-by-instruction execution.  Task t of such a job: block t / 16, row
+// (t % 16) / G of the job's rows, column group t % G; a wave's tasks (t = wave mod 8) all have column
+// group wave % G, so the wave keeps that group's slice of the activation vector in registers.
+__host__ __device__ constexpr bool joint_groups(uint32_t flags, int G, int in_dim) {
+    return (flags & MK_FLAG_JOINT_RESIDUAL) != 0 && G > 1 && 16 % G == 0 && kConsumerWaves % G == 0 &&
+           (size_t)in_dim * 2 <= sizeof(Smem::scores);
+}
+
 // Decodes the matvec instruction in queue slot `slot` (executed once per launch by one thread per
 // slot; the launch arguments come from the kernel's argument registers).
 __device__ __forceinline__ void decode_matvec(SmemPtr sm, int slot, const mk_llama_args &a) {
@@ -844,12 +873,22 @@ __device__ __forceinline__ void decode_matvec(SmemPtr sm, int slot, const mk_lla
             const int start = ins[2], end = ins[3], group = ins[4];
             const int R = a.matvec_reduction_size, in_dim = is_down ? inter : hid;
             if (start >= 0 && end <= hid / 16 && group >= 0 && group < in_dim / R && end - start <= kOutRows / 16) {
+                const int G = in_dim / R;
                 d.ntasks = (end > start ? end - start : 0) * 16;
-                d.first_row = start * 16;
                 d.row_bytes = (uint32_t)in_dim * 2u;
-                // the buffer starts at this column group's first element of the layer's matrix
-                d.w0_base = (uint64_t)(uintptr_t)((is_down ? a.down_weights : a.o_weights) + (size_t)layer * hid * in_dim + (size_t)group * R);
-                d.w0_bytes = (uint32_t)(((size_t)(hid - 1) * in_dim + R) * 2);
+                const uint16_t *matrix = (is_down ? a.down_weights : a.o_weights) + (size_t)layer * hid * in_dim;
+                if (joint_groups(a.flags, G, in_dim)) {
+                    // joint execution: this job takes 16 / G rows of each of its blocks over all G column groups
+                    d.first_row = start * 16 + group * (16 / G);
+                    d.w0_base = (uint64_t)(uintptr_t)matrix;
+                    d.w0_bytes = (uint32_t)((size_t)hid * in_dim * 2);
+                    d.gate_delta = G;
+                } else {
+                    d.first_row = start * 16;
+                    // the buffer starts at this column group's first element of the layer's matrix
+                    d.w0_base = (uint64_t)(uintptr_t)(matrix + (size_t)group * R);
+                    d.w0_bytes = (uint32_t)(((size_t)(hid - 1) * in_dim + R) * 2);
+                }
             }
         } else if (opcode == 5) {
             const int n = ins[2];
@@ -895,6 +934,12 @@ __device__ __forceinline__ RowRef matvec_row(const MatvecDesc &d, int t) {
         const long long shift = (t >> 4) & 1 ? d.gate_delta : 0;
         const WeightBuffer w = {(const uint16_t *)((uintptr_t)d.w0.base + (uintptr_t)shift), d.w0.bytes};
         return RowRef{w, (uint32_t)(blk * 16 + (t & 15)) * d.row_bytes};
+    }
+    if (d.gate_delta > 0) {
+        // jointly executed column-group job: G is a power of two
+        const int G = (int)d.gate_delta, shift = __builtin_ctz((unsigned)G);
+        const int row = d.first_row + (t >> 4) * 16 + ((t & 15) >> shift);
+        return RowRef{d.w0, (uint32_t)row * d.row_bytes + (uint32_t)(t & (G - 1)) * (d.row_bytes >> shift)};
     }
     return RowRef{d.w0, (uint32_t)(d.first_row + t) * d.row_bytes};
 }
@@ -1036,15 +1081,31 @@ __device__ __forceinline__ bool control_matvec_add(const Ctx &c) {
     const int in_dim = is_down ? a.intermediate_size : hid;
     const int ngroups = in_dim / R;
     const int nblk = end > start ? end - start : 0;
-    const uint16_t *vec = (is_down ? a.silu_out : a.attn_out) + (size_t)group * R;
+    // column groups executed jointly by this job (0: its own group only), as decoded
+    const int joint = uni((int)((const MK_LDS uint32_t *)&c.sm->desc[c.slot])[2]);
+    const uint16_t *vec = (is_down ? a.silu_out : a.attn_out) + (joint ? 0 : (size_t)group * R);
     const int wait_row = is_down ? 4 : 2;
     const int wait_target = is_down ? a.intermediate_size / 16 : a.num_attention_heads;
     uint16_t *resid = a.hidden_states;
+    // One lane per pair of adjacent residual rows.  Alone, a job owns all 16 rows of its blocks; in
+    // joint execution it owns 16 / G rows of each, starting at row group * 16 / G.
+    const int rows_per_block = joint ? 16 / joint : 16;
+    const int pairs_per_block = rows_per_block / 2;
+    const int npairs = nblk * pairs_per_block;
+    auto row0_of = [&](int p) {
+        const int bi = p / pairs_per_block, rp = p % pairs_per_block;
+        return (start + bi) * 16 + (joint ? group * rows_per_block : 0) + rp * 2;
+    };
+    // index in sm->out of the first partial sum of the pair's first row (joint: G sums per row, adjacent)
+    auto out0_of = [&](int p) {
+        const int bi = p / pairs_per_block, rp = p % pairs_per_block;
+        return joint ? bi * 16 + rp * 2 * joint : p * 2;
+    };
     // The residual rows this instruction updates were last written before its dependency was
     // satisfied, so the controller can fetch them while the consumers work.
     constexpr int kPre = 2;
     uint32_t pre[kPre] = {0, 0};
-    const bool prefetched = nblk * 8 <= kPre * 64;
+    const bool prefetched = npairs <= kPre * 64;
     PollTicket ticket = {nullptr, 0, 0};
     return controller_sequence(
         c,
@@ -1053,10 +1114,24 @@ __device__ __forceinline__ bool control_matvec_add(const Ctx &c) {
             if (!poll_wait(c, ticket, true, wait_target, release)) return false;
             trace_event(c, kEvDepReady);
             if (nblk > 0) {
-                uint4 xq[KC];
-                load_xq<KC>(xq, vec, c.lane);
-                release();
-                x_to_lds<KC>(xq, c.sm, c.lane);
+                if (joint) {
+                    // all column groups' slices of the vector, into the attention score buffer (idle here)
+                    constexpr int kMaxJoint = kConsumerWaves < 4 ? kConsumerWaves : 4;
+                    uint4 xq[kMaxJoint][KC];
+#pragma unroll
+                    for (int g = 0; g < kMaxJoint; g++)
+                        if (g < joint) load_xq<KC>(xq[g], vec + (size_t)g * R, c.lane);
+                    release();
+                    MK_LDS uint32_t *dst = (MK_LDS uint32_t *)&c.sm->scores[0][0];
+#pragma unroll
+                    for (int g = 0; g < kMaxJoint; g++)
+                        if (g < joint) x_to_lds<KC>(xq[g], dst + g * (KC * 256), c.lane);
+                } else {
+                    uint4 xq[KC];
+                    load_xq<KC>(xq, vec, c.lane);
+                    release();
+                    x_to_lds<KC>(xq, c.sm, c.lane);
+                }
             }
             return true;
         },
@@ -1065,25 +1140,31 @@ __device__ __forceinline__ bool control_matvec_add(const Ctx &c) {
 #pragma unroll
                 for (int k = 0; k < kPre; k++) {
                     const int p = c.lane + k * 64;
-                    if (p < nblk * 8) pre[k] = ld_u32(resid + start * 16 + p * 2);
+                    if (p < npairs) pre[k] = ld_u32(resid + row0_of(p));
                 }
             }
         },
         [&]() {
             bool guards_data = true;
-            if (ngroups == 1) {
-                for (int p = c.lane; p < nblk * 8; p += 64) {
-                    const int row0 = start * 16 + p * 2;
+            if (ngroups == 1 || joint) {
+                // every partial sum of these rows is here: apply them in group order, each addition
+                // rounded to bf16 as the Python VM's in-place adds are (python_vm.py:59-80)
+                const int sums = joint ? joint : 1;
+                for (int p = c.lane; p < npairs; p += 64) {
+                    const int row0 = row0_of(p), o0 = out0_of(p);
                     const uint32_t h = prefetched ? (p < 64 ? pre[0] : pre[1]) : ld_u32(resid + row0);
-                    const float lo = mkm::bf16_lo(h) + c.sm->out[p * 2];
-                    const float hi = mkm::bf16_hi(h) + c.sm->out[p * 2 + 1];
+                    float lo = mkm::bf16_lo(h), hi = mkm::bf16_hi(h);
+                    for (int g = 0; g < sums; g++) {
+                        lo = mkm::round_bf16(lo + c.sm->out[o0 + g]);
+                        hi = mkm::round_bf16(hi + c.sm->out[o0 + sums + g]);
+                    }
                     st_u32(resid + row0, mkm::pack_bf16(lo, hi));
                 }
             } else {
-                // Several column groups per block.  Every group's job but the last leaves its
-                // bf16-rounded sum as a (value, tag) pair - one 8-byte store, so whoever sees the tag
-                // sees the value, and nothing has to be acknowledged or counted.  The job of the last
-                // group fetches the others' pairs until all carry this phase's tag and applies them
+                // Several column groups per block, each job on its own.  Every group's job but the last
+                // leaves its bf16-rounded sum as a (value, tag) pair - one 8-byte store, so whoever sees
+                // the tag sees the value, and nothing has to be acknowledged or counted.  The job of the
+                // last group fetches the others' pairs until all carry this phase's tag and applies them
                 // in group order, its own last: the Python VM's order.
                 uint64_t *partial = ws_partial(c);
                 const uint32_t tag = phase_tag(c, layer, is_down);
@@ -1242,13 +1323,22 @@ __device__ __forceinline__ void park_rows(const Ctx &c, MK_LDS unsigned char *sl
 // activation vector, stream the rows (Map::size in flight), leave the results in LDS, and wait until
 // the controller has sent them.  PARKED > 0: the wave's last PARKED rows were parked in `slice` by an
 // earlier request and are taken from there; the rows before them stream as usual.
+// where this wave's activation vector lies in LDS: the common buffer, or - for a jointly executed
+// column-group job - the slice of the wave's column group in the attention score buffer
+template <int KC>
+__device__ __forceinline__ const MK_LDS uint32_t *x_source(const Ctx &c, const MatvecDesc &d) {
+    if ((d.opcode == 4 || d.opcode == 6) && d.gate_delta > 0)
+        return (const MK_LDS uint32_t *)&c.sm->scores[0][0] + (c.wave & ((int)d.gate_delta - 1)) * (KC * 256);
+    return (const MK_LDS uint32_t *)c.sm->x;
+}
+
 template <int KC, class Map, int NBUF, int PARKED = 0>
 __device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&pool)[NBUF][KC], const MatvecDesc &d, int mine,
                                              MK_LDS const unsigned char *slice = nullptr) {
     constexpr int PF = Map::size;
     if (!barrier_inputs_ready(c, true)) return false;
     XPairs<KC> x;
-    if (d.ntasks > 0) x_from_lds<KC>(x, c.sm, c.lane);
+    if (d.ntasks > 0) x_from_lds<KC>(x, x_source<KC>(c, d), c.lane);
     auto consume = [&](const uint4 (&src)[KC], int i) {
         const float y = mkm::round_bf16(dot_row<KC>(src, x));
         if (c.lane == 0) c.sm->out[c.wave + i * kConsumerWaves] = y;
@@ -1344,8 +1434,7 @@ static __device__ __noinline__ int op_oproj_upgate(SmemPtr lds, int slot, int *r
     // PARK: this worker has a long wait ahead (it came here without attention work) and its up/gate
     // instruction has at most two rows per wave beyond the six buffers: those go to LDS on entry - the
     // attention score buffer is free - and up/gate then needs nothing from HBM once its dependency resolves
-    constexpr int kParked = PARK ? 2 : 0;
-    static_assert(!PARK || (size_t)kConsumerWaves * kParked * KC * 1024 <= sizeof(Smem::scores), "parked rows fit the score buffer");
+    constexpr int kParked = PARK && (size_t)kConsumerWaves * 2 * KC * 1024 <= sizeof(Smem::scores) ? 2 : 0;
     typedef BufMap<0, 1> MapO;
     typedef BufMap<2, 3, 4, 5> MapU0;        // requested on entry
     typedef BufMap<0, 1> MapU1;              // requested when O-proj is done
@@ -1562,7 +1651,7 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
     const Ctx c = make_ctx(lds, slot, ins[0]);
     constexpr int LPT = D / 8;                   // lanes per token
     constexpr int TPW = 64 / LPT;                // tokens per wave per round
-    constexpr int NSLOT = kConsumerWaves * TPW;  // tokens per workgroup round
+    constexpr int NSLOT = kAttnWaves * TPW;  // tokens per workgroup round
     constexpr int G = kGqa;
     ArgsRef a = c.sm->args;
     const SmemPtr sm = c.sm;
@@ -1605,6 +1694,15 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
         return true;
     }
 
+    if (c.wave >= kAttnWaves) {
+        // consumer waves beyond the eight that the token -> slot mapping uses: nothing to do but keep
+        // the workgroup's barriers in step
+        if (!barrier_inputs_ready(c, true)) return false;
+        wg_barrier();
+        wg_barrier();
+        wg_barrier();
+        return true;
+    }
     const int sub = c.lane % LPT;         // which 8 dims of the head this lane owns
     const int tok_in_wave = c.lane / LPT;
     const size_t tok_stride = (size_t)KVH * D;
@@ -1754,7 +1852,7 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
     {
         f32x4 m = *(const MK_LDS f32x4 *)&sm->wave_max[0][0];
 #pragma unroll
-        for (int w = 1; w < kConsumerWaves; w++) {
+        for (int w = 1; w < kAttnWaves; w++) {
             const f32x4 o = *(const MK_LDS f32x4 *)&sm->wave_max[w][0];
             m.x = fmaxf(m.x, o.x); m.y = fmaxf(m.y, o.y); m.z = fmaxf(m.z, o.z); m.w = fmaxf(m.w, o.w);
         }
@@ -1763,7 +1861,7 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
     // p = exp(s - max), once per (token, head), in place
     if (scores_fit) {
         MK_LDS float *flat = &sm->scores[0][0];
-        for (int i = c.tid; i < G * T; i += kConsumerThreads) {
+        for (int i = c.tid; i < G * T; i += kAttnThreads) {
             const int h = i & (G - 1);
             const float m = h == 0 ? hm[0] : h == 1 ? hm[1] : h == 2 ? hm[2] : hm[3];
             flat[i] = mkm::expf_exact(flat[i] - m);
@@ -1867,17 +1965,17 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
     // one head sit in one wave, which signals for that head once its own stores have landed. ----
     if (c.tid < G * D / 2) {
         const int h = c.tid / (D / 2), d = (c.tid % (D / 2)) * 2;
-        float o0[kConsumerWaves], o1[kConsumerWaves], l[kConsumerWaves];
+        float o0[kAttnWaves], o1[kAttnWaves], l[kAttnWaves];
 #pragma unroll
-        for (int w = 0; w < kConsumerWaves; w++) {
+        for (int w = 0; w < kAttnWaves; w++) {
             o0[w] = sm->wave_o[w][h][d];
             o1[w] = sm->wave_o[w][h][d + 1];
             l[w] = sm->wave_l[w][h];
         }
 #pragma unroll
-        for (int st = 1; st < kConsumerWaves; st <<= 1)
+        for (int st = 1; st < kAttnWaves; st <<= 1)
 #pragma unroll
-            for (int i = 0; i < kConsumerWaves; i += 2 * st) {
+            for (int i = 0; i < kAttnWaves; i += 2 * st) {
                 o0[i] = o0[i] + o0[i + st];
                 o1[i] = o1[i] + o1[i + st];
                 l[i] = l[i] + l[i + st];

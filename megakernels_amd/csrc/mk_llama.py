@@ -61,6 +61,9 @@ record_timings = False
 # per-GPU array and this module allocates nothing for a launch
 static_scratch = False
 _static_scratch_ptrs: dict[int, int] = {}
+# MK_FLAG_JOINT_RESIDUAL for launches that do not say (`joint_residual=` of mk_llama): None = set it
+# when the instruction tensor qualifies, False = never (every column-group job runs on its own)
+joint_residual_default = None
 
 
 def load_library():
@@ -113,6 +116,31 @@ def _token_pointer(t, name, count=1):
     return t.data_ptr()
 
 
+def complete_residual_sets(instructions: torch.Tensor, hidden: int, inter: int, reduction: int) -> bool:
+    """Whether the column-group jobs of the residual projections (opcodes 4 and 6) come in complete
+    sets: every (opcode, layer, row block) that occurs in ``instructions`` occurs exactly once for
+    every column group.  That is what ``MK_FLAG_JOINT_RESIDUAL`` promises the kernel.  The answer is
+    kept on the tensor object (and dropped when the tensor is written to)."""
+    cached = getattr(instructions, "_mk_complete_residual_sets", None)
+    if cached is not None and cached[0] == instructions._version:
+        return cached[1]
+    words = instructions.detach().cpu().reshape(-1, instructions.shape[-1]).numpy()
+    complete = True
+    for opcode, in_dim in ((4, hidden), (6, inter)):
+        groups = in_dim // reduction
+        rows = words[words[:, 0] == opcode]
+        if groups <= 1 or len(rows) == 0:
+            continue
+        seen: dict[tuple[int, int], list[int]] = {}
+        for layer, start, end, group in rows[:, 1:5].tolist():
+            for block in range(start, end):
+                seen.setdefault((layer, block), []).append(group)
+        if any(sorted(found) != list(range(groups)) for found in seen.values()):
+            complete = False
+    instructions._mk_complete_residual_sets = (instructions._version, complete)
+    return complete
+
+
 def mk_llama(
     barriers, instructions, timings,
     qkv_weights, attn_norm_weights, o_weights, mlp_norm_weights,
@@ -124,6 +152,7 @@ def mk_llama(
     stream=None,
     *,
     embed_table=None, token_in=None, token_out=None, reset_barriers=False, num_steps=1,
+    joint_residual=None,
 ):
     """Launch one decode step asynchronously on ``stream`` (a torch stream;
     default: the current one).  Shapes are taken from the tensors.
@@ -136,7 +165,10 @@ def mk_llama(
     ``barriers`` zeroed for the next launch.  ``num_steps`` > 1 runs that many
     decode steps in the one launch: step ``s`` works at position ``pos_id + s``
     from the token of step ``s - 1`` and writes ``token_out[s]`` (``token_out``
-    then has ``num_steps`` elements)."""
+    then has ``num_steps`` elements).  ``joint_residual`` sets or clears
+    ``MK_FLAG_JOINT_RESIDUAL`` (the column-group jobs of a residual projection
+    share their rows instead of exchanging partial sums); by default the
+    instruction tensor is inspected once and the flag set when it qualifies."""
     lib = load_library()
     bf, f32, i32 = torch.bfloat16, torch.float32, torch.int32
     a = MkLlamaArgs()
@@ -213,7 +245,12 @@ def mk_llama(
         a.workspace = ws.data_ptr()
         a.workspace_bytes = ws.numel() * 4
     a.spin_limit_us = int(spin_limit_us)
-    a.flags = (1 if (record_timings and timings is not None) else 0) | (2 if reset_barriers else 0)
+    if joint_residual is None:
+        joint_residual = joint_residual_default
+    if joint_residual is None:
+        joint_residual = complete_residual_sets(instructions, hidden, inter, reduction)
+    a.flags = ((1 if (record_timings and timings is not None) else 0) | (2 if reset_barriers else 0)
+               | (4 if joint_residual else 0))
     if token_in is not None:
         if embed_table is None or tuple(embed_table.shape) != (vocab, hidden):
             raise RuntimeError("token_in needs embed_table of shape [vocab, hidden]")

@@ -52,7 +52,7 @@ def test_workspace_size_and_static_queries():
     assert small == 4 * (32 + 4 * 16 * 16 * 4 + 2 * 1024 + 2 * 4 * 2048 + 16 * 2 * 48 * 32)
     assert big > small and big < (5 << 18)
     assert lib.mk_llama_workspace_bytes(0, 2048, 8192, 2048) == 0
-    assert lib.mk_llama_query(3) == 5                      # ABI version
+    assert lib.mk_llama_query(3) == 6                      # ABI version
     assert lib.mk_llama_query(2) == 576                    # 8 consumer waves + 1 controller wave
     assert 80 * 1024 < lib.mk_llama_query(1) <= 160 * 1024  # one workgroup per CU, within gfx950's LDS
     assert lib.mk_llama_query(4) >= 2048

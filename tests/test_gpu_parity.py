@@ -88,6 +88,25 @@ def test_8b_slice_split_kv():
     _one_step_case(config_8b_slice(), workers=256, pos=1500, partitions=8, max_len=2048)
 
 
+@pytest.mark.parametrize("shape", ["tiny", "1b", "8b"])
+def test_column_group_jobs_alone_and_jointly(shape):
+    """The residual projections' column-group jobs give the checker's bits both ways: each job on its
+    own (partial sums handed to the last group's job) and, the default for complete schedules, jointly
+    (the jobs of a block share its rows).  tiny: 2 down-projection groups; 1b: 4; 8b slice: 2
+    O-projection groups run jointly, 3 down-projection groups cannot (3 does not divide 16)."""
+    import sys
+    from megakernels_amd.mk import get_mk_module
+
+    mk_mod = get_mk_module()
+    cfg, workers = {"tiny": (config_tiny(), 16), "1b": (config_1b_slice(), 256), "8b": (config_8b_slice(), 256)}[shape]
+    try:
+        for mode in (False, None):
+            mk_mod.joint_residual_default = mode
+            _one_step_case(cfg, workers=workers, pos=45)
+    finally:
+        mk_mod.joint_residual_default = None
+
+
 def _suffix_case(cfg, workers, pos, start_after_op, partitions=1):
     """The reference's diff_test `start_after_op` (scripts/diff_test.py:122-152,198-208): the first part
     of a layer is run by the checker on both sets of buffers, the megakernel then gets only the

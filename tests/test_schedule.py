@@ -245,3 +245,38 @@ def test_reduction_tree_schedule(P):
     assert all(len(serialize_and_pad(i)) == 32 for i in reds)
     kinds = [i.opcode() for i in ins]
     assert kinds.index(4) > max(j for j, k in enumerate(kinds) if k == 3)
+
+
+def test_complete_residual_sets_is_what_the_joint_flag_promises():
+    """The launch shim sets MK_FLAG_JOINT_RESIDUAL only when every (projection, layer, row block) in the
+    instruction tensor has the jobs of all its column groups, each once."""
+    import importlib
+    import sys
+
+    from megakernels_amd.mk import DEFAULT_MK_DIR
+
+    sys.path.append(str(DEFAULT_MK_DIR))
+    shim = importlib.import_module("mk_llama")
+    cfg = cfg_1b(2)
+    for workers in (132, 256):
+        sched = build(cfg, workers)
+        queues = assign_to_sms("rr", schedule=sched)
+        tensorize_instructions(sched.globs, queues)
+        words = sched.globs.instructions
+        assert shim.complete_residual_sets(words, 2048, 8192, 2048)
+        # the cached answer goes when the tensor is written to: drop one down-projection job
+        w, s = [(w, s) for w in range(words.shape[0]) for s in range(words.shape[1]) if words[w, s, 0] == 6][3]
+        saved = words[w, s].clone()
+        words[w, s] = 0
+        assert not shim.complete_residual_sets(words, 2048, 8192, 2048)
+        # the same job twice is not a complete set either
+        words[w, s] = saved
+        assert shim.complete_residual_sets(words, 2048, 8192, 2048)
+        spare = [(w2, s2) for w2 in range(words.shape[0]) for s2 in range(words.shape[1]) if words[w2, s2, 0] == 0]
+        if spare:
+            words[spare[0]] = saved
+            assert not shim.complete_residual_sets(words, 2048, 8192, 2048)
+    # a single column group (O projection of the 1B shape) never needs the promise
+    only_o = torch.zeros(4, 2, 32, dtype=torch.int32)
+    only_o[0, 0, :5] = torch.tensor([4, 0, 0, 1, 0])
+    assert shim.complete_residual_sets(only_o, 2048, 8192, 2048)
