@@ -51,22 +51,43 @@ extern "C" {
  * divides 8; other shapes run each job on its own regardless. */
 #define MK_FLAG_JOINT_RESIDUAL 4u
 
-/* Words of one instruction's timing record.  Words 0 and 4 are the reference's
- * TEVENT_CONTROLLER_START and TEVENT_CONTROLLER_END (include/util.cuh:215-219).  Words 1-3 are
- * instruction fetch done, page allocation done and semaphore set-up in the reference - stages this
- * kernel does not have (the queue is in LDS, there are no pages or semaphores) - and hold the stages
- * it has instead.  The reference's loader / consumer / storer events (words 5-54,
- * include/util.cuh:220-239) are not written by the kernel; megakernels_amd/scripts/timeline.py
- * fills them from these five on the host for tools that read the reference's layout.
- * For every executed instruction START <= DEPENDENCY_READY <= INPUT_READY <= COMPUTE_DONE <= END. */
+/* Words of one instruction's timing record: the reference's event slots (include/util.cuh:215-246),
+ * stamped by the wave that does the thing - the controller wave, the waves that stream weight rows
+ * (or K / V rows), the wave that stores and signals - so the reference's tools read measured times.
+ * Words 1-3 are instruction fetch done, page allocation done and semaphore set-up in the reference:
+ * stages this kernel does not have (the queue is in LDS, there are no pages or semaphores); they
+ * hold the controller's view of the stages it has instead.  All times are the low 32 bits of the
+ * device-wide 100 MHz clock.  For every executed instruction
+ * START <= DEPENDENCY_READY <= INPUT_READY <= COMPUTE_DONE <= END (in attention the waves that store
+ * signal on their own, so OUTPUT_READY can follow END there).  Words not listed stay as the
+ * caller left them. */
 enum {
-    MK_TIMING_START = 0,            /* the controller wave took the instruction */
+    MK_TIMING_START = 0,            /* TEVENT_CONTROLLER_START: the controller wave took the instruction */
     MK_TIMING_DEPENDENCY_READY = 1, /* the barrier counters it waits for reached their targets */
     MK_TIMING_INPUT_READY = 2,      /* activation vector normalised and handed to the consumer waves */
     MK_TIMING_COMPUTE_DONE = 3,     /* all rows of the instruction computed */
-    MK_TIMING_END = 4,              /* results stored and signalled */
-    MK_TIMING_OPCODE = 5            /* the instruction's opcode, not a time */
+    MK_TIMING_END = 4,              /* TEVENT_CONTROLLER_END: results stored and signalled, the workgroup moves on */
+    MK_TIMING_LOADER_START = 5,     /* TEVENT_LOADER_START: first weight (or K / V) row requested, by wave 0 */
+    MK_TIMING_LAUNCHER_START = 7,   /* TEVENT_LAUNCHER_START: = INPUT_READY */
+    MK_TIMING_STORER_START = 9,     /* TEVENT_STORER_START: = AT_GMEM_STORE */
+    MK_TIMING_CONSUMER_START = 11,  /* TEVENT_CONSUMER_START + 2 w, + 2 w + 1: consumer wave w starts on its
+                                       first row / is done with its last, w < MK_TIMING_CONSUMER_WAVES */
+    MK_TIMING_AT_GMEM_WAIT = 44,    /* TEVENT_AT_GMEM_WAIT: first look at the dependency counters is on its way */
+    MK_TIMING_DONE_GMEM_WAIT = 45,  /* TEVENT_DONE_GMEM_WAIT: = DEPENDENCY_READY */
+    MK_TIMING_AT_GMEM_STORE = 46,   /* TEVENT_AT_GMEM_STORE: epilogue computed, result stores issued */
+    MK_TIMING_DONE_GMEM_STORE = 47, /* TEVENT_DONE_GMEM_STORE: the stores are acknowledged */
+    MK_TIMING_FIRST_LOAD = 48,      /* TEVENT_FIRST_LOAD: = LOADER_START */
+    MK_TIMING_FIRST_USE = 49,       /* TEVENT_FIRST_USE: wave 0 starts on its first row */
+    MK_TIMING_FIRST_STORE = 50,     /* TEVENT_FIRST_STORE: = AT_GMEM_STORE */
+    MK_TIMING_LAST_LOAD = 51,       /* TEVENT_LAST_LOAD: wave 0 has requested its last row */
+    MK_TIMING_LAST_USE = 52,        /* TEVENT_LAST_USE: wave 0 is done with its last row */
+    MK_TIMING_LAST_STORE = 53,      /* TEVENT_LAST_STORE: = DONE_GMEM_STORE */
+    MK_TIMING_OUTPUT_READY = 54,    /* TEVENT_OUTPUT_READY: the barrier counters are signalled */
+    MK_TIMING_OPCODE = 55,          /* first free slot of the reference: the instruction's opcode, not a time */
+    MK_TIMING_ATTN_MAXIMA = 56,     /* attention: scores and their maxima done */
+    MK_TIMING_ATTN_PROBABILITIES = 57  /* attention: exponentials done */
 };
+#define MK_TIMING_CONSUMER_WAVES 8  /* consumer waves with a slot pair of their own */
 
 /* Status codes written by the kernel into the workspace and returned by
  * mk_llama_read_status(). */

@@ -423,6 +423,9 @@ struct Ctx {
     int *trace;                     // this instruction's timing row, or nullptr when tracing is off
 };
 
+// TR: the kernel instance that records timings.  The other instance knows at compile time that
+// there is no timing row, so none of the stamping code exists in it.
+template <bool TR>
 __device__ __forceinline__ Ctx make_ctx(SmemPtr sm, int slot, int opcode) {
     Ctx c;
     c.sm = sm;
@@ -433,8 +436,11 @@ __device__ __forceinline__ Ctx make_ctx(SmemPtr sm, int slot, int opcode) {
     c.worker = (int)blockIdx.x;
     c.slot = slot;
     c.opcode = opcode;
-    int *const rows = uni(sm->k.trace_base);
-    c.trace = rows ? rows + (size_t)(uni(sm->window_base) + slot) * MK_TIMING_SLOTS : nullptr;
+    c.trace = nullptr;
+    if constexpr (TR) {
+        int *const rows = uni(sm->k.trace_base);
+        c.trace = rows ? rows + (size_t)(uni(sm->window_base) + slot) * MK_TIMING_SLOTS : nullptr;
+    }
     return c;
 }
 
@@ -455,9 +461,66 @@ enum {
     kEvComputeDone = MK_TIMING_COMPUTE_DONE, kEvEnd = MK_TIMING_END, kEvOpcode = MK_TIMING_OPCODE
 };
 
+// stamp by the controller wave
 __device__ __forceinline__ void trace_event(const Ctx &c, int slot) {
     if (c.trace && c.controller && c.lane == 0) st_plain_i32(c.trace + slot, (int)(uint32_t)wall_clock64());
 }
+// the same moment in two slots (a stage of this kernel that is also one of the reference's events)
+__device__ __forceinline__ void trace_event(const Ctx &c, int slot, int also) {
+    if (c.trace && c.controller && c.lane == 0) {
+        const int now = (int)(uint32_t)wall_clock64();
+        st_plain_i32(c.trace + slot, now);
+        st_plain_i32(c.trace + also, now);
+    }
+}
+// stamp by whichever wave calls it (the waves that stream rows, or that store in attention)
+__device__ __forceinline__ void trace_wave(const Ctx &c, int slot) {
+    if (c.trace && c.lane == 0) st_plain_i32(c.trace + slot, (int)(uint32_t)wall_clock64());
+}
+// a consumer wave starts on its first row / is done with its last (one pair of slots per wave); wave 0
+// also stands for the instruction's first and last use of a weight row
+__device__ __forceinline__ void trace_consumer_first_use(const Ctx &c) {
+    if (c.trace && c.lane == 0 && c.wave < MK_TIMING_CONSUMER_WAVES) {
+        const int now = (int)(uint32_t)wall_clock64();
+        st_plain_i32(c.trace + MK_TIMING_CONSUMER_START + 2 * c.wave, now);
+        if (c.wave == 0) st_plain_i32(c.trace + MK_TIMING_FIRST_USE, now);
+    }
+}
+__device__ __forceinline__ void trace_consumer_last_use(const Ctx &c) {
+    if (c.trace && c.lane == 0 && c.wave < MK_TIMING_CONSUMER_WAVES) {
+        const int now = (int)(uint32_t)wall_clock64();
+        st_plain_i32(c.trace + MK_TIMING_CONSUMER_START + 2 * c.wave + 1, now);
+        if (c.wave == 0) st_plain_i32(c.trace + MK_TIMING_LAST_USE, now);
+    }
+}
+// wave 0 requested the instruction's first / its own last weight row
+__device__ __forceinline__ void trace_first_load(const Ctx &c) {
+    if (c.trace && c.lane == 0 && c.wave == 0) {
+        const int now = (int)(uint32_t)wall_clock64();
+        st_plain_i32(c.trace + MK_TIMING_LOADER_START, now);
+        st_plain_i32(c.trace + MK_TIMING_FIRST_LOAD, now);
+    }
+}
+__device__ __forceinline__ void trace_last_load(const Ctx &c) {
+    if (c.trace && c.lane == 0 && c.wave == 0) st_plain_i32(c.trace + MK_TIMING_LAST_LOAD, (int)(uint32_t)wall_clock64());
+}
+// epilogue stages of the wave that stores and signals
+__device__ __forceinline__ void trace_store_issue(const Ctx &c) {
+    if (c.trace && c.lane == 0) {
+        const int now = (int)(uint32_t)wall_clock64();
+        st_plain_i32(c.trace + MK_TIMING_STORER_START, now);
+        st_plain_i32(c.trace + MK_TIMING_AT_GMEM_STORE, now);
+        st_plain_i32(c.trace + MK_TIMING_FIRST_STORE, now);
+    }
+}
+__device__ __forceinline__ void trace_store_done(const Ctx &c) {
+    if (c.trace && c.lane == 0) {
+        const int now = (int)(uint32_t)wall_clock64();
+        st_plain_i32(c.trace + MK_TIMING_DONE_GMEM_STORE, now);
+        st_plain_i32(c.trace + MK_TIMING_LAST_STORE, now);
+    }
+}
+__device__ __forceinline__ void trace_signalled(const Ctx &c) { trace_wave(c, MK_TIMING_OUTPUT_READY); }
 
 __device__ __forceinline__ int *bar_ptr(const Ctx &c, int layer, int row, int col) {
     return uni(c.sm->args.barriers) + ((size_t)layer * MK_BARRIER_ROWS + row) * uni(c.sm->k.cols) + col;
@@ -737,6 +800,7 @@ __device__ __forceinline__ bool controller_sequence(const Ctx &c, Ahead ahead, P
     // after the controller has requested the activation vector.  A worker that arrives late then
     // has its short critical requests ahead of its own prefetch instead of behind it.
     ahead();
+    trace_event(c, MK_TIMING_AT_GMEM_WAIT);
     bool released = false;
     auto release = [&]() {
         if (!released) wg_barrier();
@@ -744,7 +808,7 @@ __device__ __forceinline__ bool controller_sequence(const Ctx &c, Ahead ahead, P
     };
     const bool ok = prepare(release);
     release();
-    trace_event(c, kEvInputReady);
+    trace_event(c, kEvInputReady, MK_TIMING_LAUNCHER_START);
     if (!barrier_inputs_ready(c, ok)) return false;
     overlap();  // runs while the consumers stream rows: fetch what the epilogue will need
     wg_barrier();
@@ -777,11 +841,13 @@ __device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need
         if (c.lane == 0) c.sm->out[c.wave + i * kConsumerWaves] = y;
     };
     wg_barrier();  // entry: the controller's first requests are out
+    trace_first_load(c);
 #pragma unroll
     for (int s = 0; s < PF; s++) request(buf[s], s);
     if (!barrier_inputs_ready(c, true)) return false;
     XPairs<KC> x;
     if (need_x) x_from_lds<KC>(x, c.sm, c.lane);
+    trace_consumer_first_use(c);
     int base = 0;
     // rounds that are followed by more rows: every row of the round exists, every slot is refilled
     for (; base + PF < mine; base += PF) {
@@ -793,10 +859,12 @@ __device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need
             compiler_fence();
         }
     }
+    trace_last_load(c);
     // last round: nothing left to request
 #pragma unroll
     for (int s = 0; s < PF; s++)
         if (base + s < mine) consume(buf[s], base + s, x);
+    trace_consumer_last_use(c);
     wg_barrier();
     // hold the next instruction's weight requests back until the controller has sent this
     // instruction's results and signal: they would otherwise queue behind the bulk loads
@@ -970,7 +1038,7 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
         },
         [&](auto release) {
             if (layer > 0 && !poll_wait(c, ticket, true, down_jobs, release)) return false;
-            trace_event(c, kEvDepReady);
+            trace_event(c, kEvDepReady, MK_TIMING_DONE_GMEM_WAIT);
             if (nblk > 0) {
                 // layer 0 of a launch that was given a token reads the embedding row itself; the
                 // worker holding the first block also makes it the residual stream (every later
@@ -1051,9 +1119,12 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
                     emit(p, c0, c1, s0, s1);
                 }
             }
+            trace_store_issue(c);
             wait_stores();
+            trace_store_done(c);
             // one arrival per block on its head's counter (python_vm.py:248)
             for (int b = c.lane; b < nblk; b += 64) add_i32(pad_ptr(c, layer, 0, (start + b) / (D / 16)), 1);
+            trace_signalled(c);
         });
 }
 
@@ -1112,7 +1183,7 @@ __device__ __forceinline__ bool control_matvec_add(const Ctx &c) {
         [&]() { ticket = poll_issue(c, sharded_lane_ptr(c, layer, wait_row)); },
         [&](auto release) {
             if (!poll_wait(c, ticket, true, wait_target, release)) return false;
-            trace_event(c, kEvDepReady);
+            trace_event(c, kEvDepReady, MK_TIMING_DONE_GMEM_WAIT);
             if (nblk > 0) {
                 if (joint) {
                     // all column groups' slices of the vector, into the attention score buffer (idle here)
@@ -1217,8 +1288,11 @@ __device__ __forceinline__ bool control_matvec_add(const Ctx &c) {
             }
             // an arrival that stands for nothing another worker reads (a partial sum carries its own
             // tag) need not wait for its stores
+            trace_store_issue(c);
             if (guards_data) wait_stores();
+            trace_store_done(c);
             signal_sharded(c, layer, is_down ? 5 : 3, nblk);
+            trace_signalled(c);
         });
 }
 
@@ -1243,7 +1317,7 @@ __device__ __forceinline__ bool control_upgate(const Ctx &c) {
         },
         [&](auto release) {
             if (!poll_wait(c, ticket, true, o_jobs, release)) return false;
-            trace_event(c, kEvDepReady);
+            trace_event(c, kEvDepReady, MK_TIMING_DONE_GMEM_WAIT);
             if (n > 0) {
                 XVec<KC> x;
                 load_x<KC>(x, a.hidden_states, c.lane);
@@ -1264,8 +1338,11 @@ __device__ __forceinline__ bool control_upgate(const Ctx &c) {
                 const float s1 = mkm::round_bf16(mkm::silu_exact(gate[r + 1]));
                 st_u32(a.silu_out + ins[3 + i] * 16 + r, mkm::pack_bf16(s0 * up[r], s1 * up[r + 1]));
             }
+            trace_store_issue(c);
             wait_stores();
+            trace_store_done(c);
             signal_sharded(c, layer, 4, n);
+            trace_signalled(c);
         });
 }
 
@@ -1339,6 +1416,7 @@ __device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&pool)[NBUF][K
     if (!barrier_inputs_ready(c, true)) return false;
     XPairs<KC> x;
     if (d.ntasks > 0) x_from_lds<KC>(x, x_source<KC>(c, d), c.lane);
+    trace_consumer_first_use(c);
     auto consume = [&](const uint4 (&src)[KC], int i) {
         const float y = mkm::round_bf16(dot_row<KC>(src, x));
         if (c.lane == 0) c.sm->out[c.wave + i * kConsumerWaves] = y;
@@ -1357,6 +1435,7 @@ __device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&pool)[NBUF][K
             compiler_fence();
         }
     }
+    trace_last_load(c);
     // last round: nothing left to request
 #pragma unroll
     for (int s = 0; s < PF; s++)
@@ -1375,6 +1454,7 @@ __device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&pool)[NBUF][K
                 consume(row, parked_first + r);
             }
     }
+    trace_consumer_last_use(c);
     wg_barrier();  // results are in LDS
     // hold further weight requests back until the controller has sent this instruction's results and
     // signal: they would otherwise queue behind the bulk loads
@@ -1405,17 +1485,18 @@ template <> struct FirstBuffers<5> { typedef BufMap<0, 1, 2, 3, 4> type; };
 template <> struct FirstBuffers<6> { typedef BufMap<0, 1, 2, 3, 4, 5> type; };
 
 // One matvec instruction (opcode OP, row width KC chunks).
-template <int OP, int KC, int PARKED = 0>
+template <bool TR, int OP, int KC, int PARKED = 0>
 static __device__ __noinline__ bool op_matvec(SmemPtr lds, int slot, int *refusal) {
     constexpr int PF = rows_in_flight<KC>(pf_of(OP));
     typedef typename FirstBuffers<PF>::type Map;
-    const Ctx c = make_ctx(lds, slot, OP);
+    const Ctx c = make_ctx<TR>(lds, slot, OP);
     MatvecDesc d;
     if (!describe_matvec(lds, slot, OP, d)) return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
     if (c.controller) return control_matvec<KC>(c);
     const int mine = rows_of_wave(d.ntasks, c.wave);
     uint4 pool[PF][KC];
     wg_barrier();  // entry: the controller's first requests are out
+    trace_first_load(c);
     request_rows<KC, Map>(c, pool, d, 0, mine > PARKED ? mine - PARKED : 0);
     const bool ok = consumer_run<KC, Map, PF, PARKED>(c, pool, d, mine, (MK_LDS const unsigned char *)lds->park + c.wave * (KC * 1024));
     return ok;
@@ -1428,7 +1509,7 @@ static __device__ __noinline__ bool op_matvec(SmemPtr lds, int slot, int *refusa
 // are requested together with the O-proj rows, and the two O-proj buffers go to up/gate as soon as
 // O-proj is done.  Returns the number of instructions executed (2, or 1 when the second instruction
 // is malformed and left to report itself), 0 on failure.
-template <int KC, bool PARK>
+template <bool TR, int KC, bool PARK>
 static __device__ __noinline__ int op_oproj_upgate(SmemPtr lds, int slot, int *refusal) {
     constexpr int NBUF = 6;
     // PARK: this worker has a long wait ahead (it came here without attention work) and its up/gate
@@ -1439,8 +1520,8 @@ static __device__ __noinline__ int op_oproj_upgate(SmemPtr lds, int slot, int *r
     typedef BufMap<2, 3, 4, 5> MapU0;        // requested on entry
     typedef BufMap<0, 1> MapU1;              // requested when O-proj is done
     typedef BufMap<2, 3, 4, 5, 0, 1> MapU;
-    const Ctx co = make_ctx(lds, slot, 4);
-    const Ctx cu = make_ctx(lds, slot + 1, 5);
+    const Ctx co = make_ctx<TR>(lds, slot, 4);
+    const Ctx cu = make_ctx<TR>(lds, slot + 1, 5);
     MatvecDesc dso, dsu;
     if (!describe_matvec(lds, slot, 4, dso)) {
         bail(co, MK_STATUS_BAD_INSTRUCTION, refusal);
@@ -1461,7 +1542,9 @@ static __device__ __noinline__ int op_oproj_upgate(SmemPtr lds, int slot, int *r
     const int stream_u = mine_u > kParked ? mine_u - kParked : 0;  // up/gate rows that go through the buffers
     uint4 pool[NBUF][KC];
     wg_barrier();  // entry of O-proj: the controller's first requests are out
+    trace_first_load(co);
     request_rows<KC, MapO>(co, pool, dso, 0, mine_o);
+    if (pair) trace_first_load(cu);
     request_rows<KC, MapU0>(co, pool, dsu, 0, stream_u, pair);
     MK_LDS unsigned char *slice = (MK_LDS unsigned char *)&lds->scores[0][0] + co.wave * (kParked * KC * 1024);
     if constexpr (PARK) {
@@ -1500,10 +1583,10 @@ __device__ __forceinline__ void argmax_combine_wave(float &v, int &i) {
 // opcode 7: final RMSNorm + LM head  (python_vm.py:251-274;
 // reference device op: demos/low-latency-llama/rms_lm_head.cu:10-117)
 // ---------------------------------------------------------------------------------------------
-template <int KC>
+template <bool TR, int KC>
 static __device__ __noinline__ bool op_lm_head(SmemPtr lds, int slot, int *refusal) {
     const InsPtr ins = lds->queue[slot];
-    const Ctx c = make_ctx(lds, slot, ins[0]);
+    const Ctx c = make_ctx<TR>(lds, slot, ins[0]);
     ArgsRef a = c.sm->args;
     const int start = ins[1], end = ins[2];
     const int hid = a.hidden_size;
@@ -1530,7 +1613,7 @@ static __device__ __noinline__ bool op_lm_head(SmemPtr lds, int slot, int *refus
             [&](auto release) {
                 if (!first) return true;  // the activation vector stays in LDS between batches
                 if (!poll_wait(c, ticket, true, down_jobs, release)) return false;
-                trace_event(c, kEvDepReady);
+                trace_event(c, kEvDepReady, MK_TIMING_DONE_GMEM_WAIT);
                 XVec<KC> x;
                 load_x<KC>(x, a.hidden_states, c.lane);
                 release();
@@ -1549,6 +1632,7 @@ static __device__ __noinline__ bool op_lm_head(SmemPtr lds, int slot, int *refus
                     if (y0 > best_v) { best_v = y0; best_i = row; }
                     if (y1 > best_v) { best_v = y1; best_i = row + 1; }
                 }
+                trace_store_issue(c);
             });
         if (!ok) return false;
         first = false;
@@ -1645,10 +1729,10 @@ __device__ __forceinline__ MergedPair merge_partitions(const Ctx &c, int head, i
 // tokens in increasing order and slots are combined by a pairwise tree (token groups of a wave,
 // then waves).  A token's row is spread over D/8 lanes, 8 dims each.
 // ---------------------------------------------------------------------------------------------
-template <int D>
+template <bool TR, int D>
 static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *refusal) {
     const InsPtr ins = lds->queue[slot];
-    const Ctx c = make_ctx(lds, slot, ins[0]);
+    const Ctx c = make_ctx<TR>(lds, slot, ins[0]);
     constexpr int LPT = D / 8;                   // lanes per token
     constexpr int TPW = 64 / LPT;                // tokens per wave per round
     constexpr int NSLOT = kAttnWaves * TPW;  // tokens per workgroup round
@@ -1680,15 +1764,14 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
         const bool mine = c.lane < G + 2;
         const bool ok = poll_counters(c, mine ? pad_ptr(c, layer, 0, col) : nullptr, mine ? bar_ptr(c, layer, 0, col) : nullptr,
                                       false, D / 16);
-        trace_event(c, kEvDepReady);
+        trace_event(c, kEvDepReady, MK_TIMING_DONE_GMEM_WAIT);
         if (!barrier_inputs_ready(c, ok)) return false;
         trace_event(c, kEvInputReady);
         wg_barrier();  // wave maxima
-        trace_event(c, 6);
+        trace_event(c, MK_TIMING_ATTN_MAXIMA);
         wg_barrier();  // probabilities
-        trace_event(c, 7);
+        trace_event(c, MK_TIMING_ATTN_PROBABILITIES);
         wg_barrier();  // wave sums
-        trace_event(c, 8);
         trace_event(c, kEvComputeDone);
         // the waves that combine the sums store and signal on their own
         return true;
@@ -1724,6 +1807,7 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
     // the dependency is known.
     constexpr int RU = 4;
     uint4 kraw[RU], vraw[RU];
+    trace_first_load(c);
 #pragma unroll
     for (int u = 0; u < RU; u++) {
         const int r = token_of(u);
@@ -1735,6 +1819,7 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
     }
     if (!barrier_inputs_ready(c, true)) return false;
 
+    trace_consumer_first_use(c);
     uint4 q[G];  // this lane's 8 dims of the four query heads, as bf16 pairs
     {
 #pragma unroll
@@ -1959,6 +2044,7 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
         for (int h = 0; h < G; h++) l[h] = lane_tree_sum<LPT, 64>(lsum[h]);
         if (c.lane == 0) *(MK_LDS f32x4 *)&sm->wave_l[c.wave][0] = f32x4{l[0], l[1], l[2], l[3]};
     }
+    trace_consumer_last_use(c);
     wg_barrier();
 
     // ---- combine the 8 waves pairwise, normalise, store: thread -> (head, dim pair).  The threads of
@@ -1999,11 +2085,15 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
             st_f32(dst + 1, r1);
             if (d == 0) st_f32(a.attn_lse_intermediates + (size_t)head * a.max_partials + pidx, lse);
         }
+        // (the stamps of the storing waves share their slots: the last wave to get there is on record)
+        trace_store_issue(c);
         wait_stores();
+        trace_store_done(c);
         if (d == 0) {
             if (skip) signal_sharded_lane(c, layer, 2, 1);
             else add_i32(pad_ptr(c, layer, 1, head), 1);
         }
+        trace_signalled(c);
     }
     return true;
 }
@@ -2012,10 +2102,10 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
 // opcode 3: log-sum-exp merge of attention partitions  (python_vm.py:349-393;
 // reference device op: demos/low-latency-llama/attention_reduction.cu:18-339)
 // ---------------------------------------------------------------------------------------------
-template <int D>
+template <bool TR, int D>
 static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot, int *refusal) {
     const InsPtr ins = lds->queue[slot];
-    const Ctx c = make_ctx(lds, slot, ins[0]);
+    const Ctx c = make_ctx<TR>(lds, slot, ins[0]);
     ArgsRef a = c.sm->args;
     constexpr int kMaxList = MK_INSTRUCTION_WORDS - 7;
     constexpr int TPH = D / 2;  // threads per head, two output dims each; all in one wave
@@ -2042,6 +2132,11 @@ static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot
         const PollTicket ticket =
             poll_issue(c, leader ? pad_ptr(c, layer, 1, head) : nullptr, leader ? bar_ptr(c, layer, 1, head) : nullptr);
         if (poll_wait(c, ticket, false, P, []() {})) {
+            if (c.wave == 0) {
+                trace_wave(c, kEvDepReady);
+                trace_wave(c, MK_TIMING_DONE_GMEM_WAIT);
+            }
+            trace_consumer_first_use(c);
             const MergedPair r = merge_partitions<D>(c, head, j, n, [&](int k) { return ins[6 + k]; });
             if (terminal) {
                 st_u32(a.attn_out + (size_t)head * D + d, mkm::pack_bf16(r.o0, r.o1));
@@ -2051,7 +2146,10 @@ static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot
                 st_f32(dst + 1, r.o1);
                 if (leader) st_f32(a.attn_lse_intermediates + (size_t)head * MP + out_idx, r.lse);
             }
+            trace_consumer_last_use(c);
+            trace_store_issue(c);
             wait_stores();
+            trace_store_done(c);
             // A terminal merge completes the head for the O projection (barrier row 2).  A merge
             // inside a reduction tree is one more arrival among the head's partial results (row 1):
             // the merge that consumes it waits for the partitions plus the merges below it.
@@ -2059,12 +2157,14 @@ static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot
                 if (terminal) signal_sharded_lane(c, layer, 2, 1);
                 else add_i32(pad_ptr(c, layer, 1, head), 1);
             }
+            trace_signalled(c);
         } else if (c.lane == 0) {
             c.sm->abort = 1;
         }
     }
+    if (c.controller) trace_event(c, MK_TIMING_AT_GMEM_WAIT);
     wg_barrier();
-    trace_event(c, kEvDepReady);
+    // (the first merging wave stamped the moment it saw its heads' partitions complete)
     trace_event(c, kEvInputReady);
     trace_event(c, kEvComputeDone);
     return c.sm->abort == 0;
@@ -2073,7 +2173,7 @@ static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot
 // ---------------------------------------------------------------------------------------------
 // the persistent kernel
 // ---------------------------------------------------------------------------------------------
-template <int KC_HID, int KC_RED, int D>
+template <int KC_HID, int KC_RED, int D, bool TR>
 __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args a) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     const SmemPtr sm = (SmemPtr)smem_raw;
@@ -2145,7 +2245,7 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
     int refusal = 0;
     if (a.token_in && sm->token < 0) {
         // every workgroup sees the same bad token and skips its queue
-        if (tid == kConsumerThreads) record_status(make_ctx(sm, 0, 0), MK_STATUS_BAD_TOKEN);
+        if (tid == kConsumerThreads) record_status(make_ctx<TR>(sm, 0, 0), MK_STATUS_BAD_TOKEN);
         refusal = MK_STATUS_BAD_TOKEN;
     }
     // A launch covers one decode step, or `num_steps` of them back to back: the token a step
@@ -2164,15 +2264,15 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
             const int opcode = sm->queue[slot][0];
             if (opcode == 0) continue;  // NoOp pads the queues (megakernels/scheduler.py:287-289)
             {
-                const Ctx c = make_ctx(sm, slot, opcode);
+                const Ctx c = make_ctx<TR>(sm, slot, opcode);
                 trace_event(c, kEvStart);
                 if (c.trace && c.controller && c.lane == 0) st_plain_i32(c.trace + kEvOpcode, opcode);
             }
             bool ok = true;
             switch (opcode) {
-            case 1: ok = op_matvec<1, KC_HID>(sm, slot, &refusal); break;
-            case 2: ok = op_attention<D>(sm, slot, &refusal); break;
-            case 3: ok = op_attention_reduction<D>(sm, slot, &refusal); break;
+            case 1: ok = op_matvec<TR, 1, KC_HID>(sm, slot, &refusal); break;
+            case 2: ok = op_attention<TR, D>(sm, slot, &refusal); break;
+            case 3: ok = op_attention_reduction<TR, D>(sm, slot, &refusal); break;
             case 4:
                 if constexpr (KC_HID == KC_RED && MK_PAIR_OPROJ_UPGATE) {
                     if (slot + 1 < window_slots && sm->queue[slot + 1][0] == 5) {
@@ -2182,30 +2282,30 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
                         // enough (two list entries: eight rows per wave)
                         const bool park = MK_PARK_UPGATE && !a.skip_attn_reduction && (slot == 0 || sm->queue[slot - 1][0] != 2) &&
                                           sm->queue[slot + 1][2] >= 0 && sm->queue[slot + 1][2] <= 2;
-                        const int executed = park ? op_oproj_upgate<KC_HID, true>(sm, slot, &refusal)
-                                                  : op_oproj_upgate<KC_HID, false>(sm, slot, &refusal);
+                        const int executed = park ? op_oproj_upgate<TR, KC_HID, true>(sm, slot, &refusal)
+                                                  : op_oproj_upgate<TR, KC_HID, false>(sm, slot, &refusal);
                         ok = executed > 0;
                         slot += ok ? executed - 1 : 0;
                         break;
                     }
                 }
-                ok = op_matvec<4, KC_RED>(sm, slot, &refusal);
+                ok = op_matvec<TR, 4, KC_RED>(sm, slot, &refusal);
                 break;
-            case 5: ok = op_matvec<5, KC_HID>(sm, slot, &refusal); break;
+            case 5: ok = op_matvec<TR, 5, KC_HID>(sm, slot, &refusal); break;
             case 6:
             if constexpr (KC_HID == KC_RED && MK_PAIR_OPROJ_UPGATE && MK_PARK_UPGATE && MK_PARK_DOWN) {
                 if (sm->parked_slot == slot) {
-                    ok = op_matvec<6, KC_RED, 1>(sm, slot, &refusal);
+                    ok = op_matvec<TR, 6, KC_RED, 1>(sm, slot, &refusal);
                     break;
                 }
             }
-            ok = op_matvec<6, KC_RED>(sm, slot, &refusal);
+            ok = op_matvec<TR, 6, KC_RED>(sm, slot, &refusal);
             break;
-            case 7: ok = op_lm_head<KC_HID>(sm, slot, &refusal); break;
-            default: ok = bail(make_ctx(sm, slot, opcode), MK_STATUS_BAD_OPCODE, &refusal);  // reference: trap, include/util.cuh:38
+            case 7: ok = op_lm_head<TR, KC_HID>(sm, slot, &refusal); break;
+            default: ok = bail(make_ctx<TR>(sm, slot, opcode), MK_STATUS_BAD_OPCODE, &refusal);  // reference: trap, include/util.cuh:38
             }
             if (!ok) break;
-            trace_event(make_ctx(sm, slot, sm->queue[slot][0]), kEvEnd);
+            trace_event(make_ctx<TR>(sm, slot, sm->queue[slot][0]), kEvEnd);
         }
         if (sm->abort) break;
       }
@@ -2342,7 +2442,7 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
                 }
                 if (published > step) break;
                 if (wall_clock64() - t0 > limit) {
-                    if (tid == 0) record_status(make_ctx(sm, 0, 0), MK_STATUS_BARRIER_TIMEOUT);
+                    if (tid == 0) record_status(make_ctx<TR>(sm, 0, 0), MK_STATUS_BARRIER_TIMEOUT);
                     ok = false;
                     break;
                 }
@@ -2417,10 +2517,10 @@ int fail(int code, const char *fmt, ...) {
 
 using KernelFn = void (*)(const mk_llama_args);
 
-KernelFn pick_kernel(int hid, int R, int D) {
-    if (hid == 2048 && R == 2048 && D == 64) return mk_llama_kernel<4, 4, 64>;
-    if (hid == 4096 && R == 2048 && D == 128) return mk_llama_kernel<8, 4, 128>;
-    if (hid == 512 && R == 512 && D == 64) return mk_llama_kernel<1, 1, 64>;
+KernelFn pick_kernel(int hid, int R, int D, bool timings) {
+    if (hid == 2048 && R == 2048 && D == 64) return timings ? mk_llama_kernel<4, 4, 64, true> : mk_llama_kernel<4, 4, 64, false>;
+    if (hid == 4096 && R == 2048 && D == 128) return timings ? mk_llama_kernel<8, 4, 128, true> : mk_llama_kernel<8, 4, 128, false>;
+    if (hid == 512 && R == 512 && D == 64) return timings ? mk_llama_kernel<1, 1, 64, true> : mk_llama_kernel<1, 1, 64, false>;
     return nullptr;
 }
 
@@ -2500,7 +2600,7 @@ int validate(const mk_llama_args &a, KernelFn *kernel) {
     // weight rows are addressed as 32-bit offsets into one buffer per matrix
     const uint64_t widest = 2ull * hid * (uint64_t)(a.vocab_size > a.intermediate_size ? a.vocab_size : a.intermediate_size);
     if (widest >= (1ull << 31)) return fail(-3, "a weight matrix of %llu bytes exceeds the 2 GiB a buffer can address", (unsigned long long)widest);
-    KernelFn fn = pick_kernel(hid, R, D);
+    KernelFn fn = pick_kernel(hid, R, D, (a.flags & MK_FLAG_TIMINGS) != 0 && a.timings != nullptr);
     if (!fn) return fail(-5, "no kernel instance for hidden %d, reduction width %d, head_dim %d", hid, R, D);
     const uint64_t need = mk_llama_workspace_bytes(a.num_layers, hid, a.intermediate_size, R);
     if (a.workspace_bytes < need)

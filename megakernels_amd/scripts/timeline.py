@@ -34,32 +34,21 @@ from megakernels_amd.utils import get_sm_count, set_sm_count_override
 
 NAMES = {1: "qkv", 2: "attention", 3: "merge", 4: "o-proj", 5: "up/gate", 6: "down", 7: "lm-head"}
 
-# The reference's event slots (include/util.cuh:215-246) and the record of this kernel (MK_TIMING_* of
-# include/mk_llama.h: 0 start, 1 dependency seen, 2 input ready, 3 rows done, 4 end) each one is taken
-# from.  The reference's stages that this kernel does not have (instruction fetch, page allocation,
-# semaphore set-up: all done before an instruction starts here) get the start time.
-REFERENCE_EVENTS = {
-    0: 0,    # TEVENT_CONTROLLER_START
-    1: 0,    # TEVENT_IFETCH_DONE
-    2: 0,    # TEVENT_PAGE_ALLOC_DONE
-    3: 0,    # TEVENT_SEMS_SETUP
-    4: 4,    # TEVENT_CONTROLLER_END
-    5: 0,    # TEVENT_LOADER_START: the first weight rows are requested on entry
-    7: 2,    # TEVENT_LAUNCHER_START
-    9: 3,    # TEVENT_STORER_START
-    11: 2,   # TEVENT_CONSUMER_START
-    44: 0,   # TEVENT_AT_GMEM_WAIT
-    45: 1,   # TEVENT_DONE_GMEM_WAIT
-    46: 3,   # TEVENT_AT_GMEM_STORE
-    47: 4,   # TEVENT_DONE_GMEM_STORE
-    48: 0,   # TEVENT_FIRST_LOAD
-    49: 2,   # TEVENT_FIRST_USE
-    50: 3,   # TEVENT_FIRST_STORE
-    51: 3,   # TEVENT_LAST_LOAD
-    52: 3,   # TEVENT_LAST_USE
-    53: 4,   # TEVENT_LAST_STORE
-    54: 4,   # TEVENT_OUTPUT_READY
-}
+# Slots of a timing record (MK_TIMING_* of include/mk_llama.h; the reference's TEVENT_* of
+# include/util.cuh:215-246 where the names agree).
+START, DEP_READY, INPUT_READY, COMPUTE_DONE, END = 0, 1, 2, 3, 4
+LOADER_START, LAUNCHER_START, STORER_START, CONSUMER_START = 5, 7, 9, 11
+AT_GMEM_WAIT, DONE_GMEM_WAIT, AT_GMEM_STORE, DONE_GMEM_STORE = 44, 45, 46, 47
+FIRST_LOAD, FIRST_USE, FIRST_STORE, LAST_LOAD, LAST_USE, LAST_STORE, OUTPUT_READY = 48, 49, 50, 51, 52, 53, 54
+OPCODE, ATTN_MAXIMA, ATTN_PROBABILITIES = 55, 56, 57
+CONSUMER_WAVES = 8
+# every slot that holds a time
+TIME_SLOTS = ([START, DEP_READY, INPUT_READY, COMPUTE_DONE, END, LOADER_START, LAUNCHER_START, STORER_START]
+              + list(range(CONSUMER_START, CONSUMER_START + 2 * CONSUMER_WAVES))
+              + list(range(AT_GMEM_WAIT, OUTPUT_READY + 1)) + [ATTN_MAXIMA, ATTN_PROBABILITIES])
+# The reference's stages that this kernel does not have (instruction fetch, page allocation, semaphore
+# set-up: the queue is in LDS, there are no pages or semaphores) are over when an instruction starts.
+REFERENCE_ONLY_STAGES = (1, 2, 3)   # TEVENT_IFETCH_DONE, TEVENT_PAGE_ALLOC_DONE, TEVENT_SEMS_SETUP
 
 
 def launch_origin(starts) -> int:
@@ -72,20 +61,36 @@ def launch_origin(starts) -> int:
 
 
 def reference_event_layout(timings: torch.Tensor, instructions: torch.Tensor) -> torch.Tensor:
-    """``timings [workers, slots, 128]`` of this kernel re-laid as the reference's tools expect them:
-    the slots of ``REFERENCE_EVENTS`` filled, as ticks (10 ns) since the first instruction of the
-    launch started; everything else zero, as are the rows of NoOp padding."""
+    """``timings [workers, slots, 128]`` as the reference's tools expect them: every event the kernel
+    stamped, in the reference's slot, as ticks (10 ns) since the first instruction of the launch
+    started; slots 1-3 (stages only the reference has) hold the start; a slot the kernel did not stamp
+    for an instruction (a wave without rows, an instruction kind without that stage) is zero, as are
+    the rows of NoOp padding.  Slot 55, the reference's first free one, keeps the opcode."""
     t = timings.cpu().to(torch.int64)
     ins = instructions.cpu()
     executed = ins[:, :, 0] != 0
     out = torch.zeros_like(t)
     if not bool(executed.any()):
         return out.to(torch.int32)
-    origin = launch_origin(t[:, :, 0][executed].numpy())
-    ticks = ((t[:, :, :5] & 0xFFFFFFFF) - origin) % (1 << 32)
-    for slot, source in REFERENCE_EVENTS.items():
-        out[:, :, slot] = torch.where(executed, ticks[:, :, source], torch.zeros_like(ticks[:, :, source]))
+    origin = launch_origin(t[:, :, START][executed].numpy())
+    for slot in TIME_SLOTS:
+        raw = t[:, :, slot]
+        ticks = ((raw & 0xFFFFFFFF) - origin) % (1 << 32)
+        out[:, :, slot] = torch.where(executed & (raw != 0), ticks, torch.zeros_like(ticks))
+    for slot in REFERENCE_ONLY_STAGES:
+        out[:, :, slot] = out[:, :, START]
+    out[:, :, OPCODE] = torch.where(executed, t[:, :, OPCODE], torch.zeros_like(t[:, :, OPCODE]))
     return out.to(torch.int32)
+
+
+def microseconds(timings: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
+    """``(t, stamped)``: the records as microseconds since the launch's first instruction started, and
+    which slots were stamped at all."""
+    raw = timings.astype(np.int64)
+    executed = raw[:, :, OPCODE] != 0
+    origin = np.int64(launch_origin(raw[:, :, START][executed]))
+    t = ((raw & 0xFFFFFFFF) - origin) % (1 << 32) / 100.0
+    return t, raw != 0
 
 
 def main(argv):
@@ -135,44 +140,60 @@ def main(argv):
     mk.record_timings = False
     mk.check_status(device)
 
-    # [workers, slots, 6]: start, dependency seen, activation ready, rows done, end, opcode
-    t = globs.timings.cpu()[:, :, :6].numpy().astype(np.float64)
+    raw = globs.timings.cpu().numpy()
     ins = globs.instructions.cpu().numpy()
-    # the records are the low 32 bits of the device clock: times since the earliest record
-    executed = t[:, :, 5] != 0
-    origin = np.int64(launch_origin(globs.timings.cpu()[:, :, 0].numpy()[executed]))
-    t[:, :, :5] = ((t[:, :, :5].astype(np.int64) - origin) % (1 << 32)) / 100.0
+    t, stamped = microseconds(raw)
+    op_of = raw[:, :, OPCODE]
     if opts["out"]:
-        np.savez_compressed(opts["out"], timings=globs.timings.cpu().numpy(), instructions=ins,
+        np.savez_compressed(opts["out"], timings=raw, instructions=ins,
                             reference_layout=reference_event_layout(globs.timings, globs.instructions).numpy(),
                             ticks_per_microsecond=np.array(100))
     print(f"{opts['model']}, {opts['layers']} layers, position {pos}, {partitions} attention partitions, {workers} workers, "
           f"assignment {opts['sched']}: kernel {start.elapsed_time(end) * 1e3:.1f} us with timing records on, "
-          f"last instruction ends at {t[:, :, 4].max():.1f} us")
-    print("\nper instruction kind, mean / max over all instructions (us):")
-    print(f"{'kind':10s} {'count':>6s} {'wait for dependency':>20s} {'activation':>14s} {'rows':>14s} {'write back':>14s}")
+          f"last instruction ends at {t[:, :, END][op_of != 0].max():.1f} us")
+    print("\nper instruction kind, mean / max over all instructions (us); the write back is split into: epilogue "
+          "computed and stores issued | stores acknowledged | signalled | workgroup moves on:")
+    print(f"{'kind':10s} {'count':>6s} {'wait for dependency':>20s} {'activation':>14s} {'rows':>14s} {'write back':>14s}"
+          f" {'issue':>13s} {'ack':>13s} {'signal':>13s} {'leave':>13s}")
+    cell = lambda a: f"{a.mean():6.2f} /{a.max():6.2f}" if a.size else "      -"
     for op, name in NAMES.items():
-        sel = t[:, :, 5] == op
+        sel = op_of == op
         if not sel.any():
             continue
-        st, dep, inp, rows, done = (t[:, :, i][sel] for i in range(5))
+        st, dep, inp, rows, done = (t[:, :, i][sel] for i in (START, DEP_READY, INPUT_READY, COMPUTE_DONE, END))
         if op in (2, 3):
             inp = dep  # these record no separate activation event
-        cell = lambda a: f"{a.mean():6.2f} /{a.max():6.2f}"
-        print(f"{name:10s} {int(sel.sum()):6d} {cell(dep - st):>20s} {cell(inp - dep):>14s} {cell(rows - inp):>14s} {cell(done - rows):>14s}")
+        line = (f"{name:10s} {int(sel.sum()):6d} {cell(dep - st):>20s} {cell(inp - dep):>14s} {cell(rows - inp):>14s} "
+                f"{cell(done - rows):>14s}")
+        full = sel & stamped[:, :, AT_GMEM_STORE] & stamped[:, :, DONE_GMEM_STORE] & stamped[:, :, OUTPUT_READY]
+        if full.any() and op not in (2, 3):
+            issue, ack, sig = (t[:, :, i][full] for i in (AT_GMEM_STORE, DONE_GMEM_STORE, OUTPUT_READY))
+            line += (f" {cell(issue - t[:, :, COMPUTE_DONE][full]):>13s} {cell(ack - issue):>13s} {cell(sig - ack):>13s} "
+                     f"{cell(t[:, :, END][full] - sig):>13s}")
+        print(line)
     layer = min(opts["layer"], opts["layers"] - 1)
-    print(f"\nlayer {layer}, over the workers that run the kind (us): first start | dependency seen p10 p50 max | end p10 p50 max")
+    q = lambda a, ps: " ".join(f"{np.percentile(a, p):7.2f}" for p in ps)
+    print(f"\nlayer {layer}, over the workers that run the kind (us): first start | dependency seen p10 p50 max | "
+          f"last row done (slowest wave) p50 max | signalled p50 max | end p50 max")
     for op in range(1, 7):
         sel = (ins[:, :, 0] == op) & (ins[:, :, 1] == layer)
         if not sel.any():
             continue
-        st, dep, done = t[:, :, 0][sel], t[:, :, 1][sel], t[:, :, 4][sel]
-        q = lambda a, ps: " ".join(f"{np.percentile(a, p):7.2f}" for p in ps)
-        print(f"  {NAMES[op]:10s} {st.min():7.2f} | {q(dep, (10, 50, 100))} | {q(done, (10, 50, 100))}")
+        st, dep, done = t[:, :, START][sel], t[:, :, DEP_READY][sel], t[:, :, END][sel]
+        waves = np.stack([np.where(stamped[:, :, CONSUMER_START + 2 * w + 1], t[:, :, CONSUMER_START + 2 * w + 1], 0.0)[sel]
+                          for w in range(CONSUMER_WAVES)]).max(axis=0)
+        sig = np.where(stamped[:, :, OUTPUT_READY], t[:, :, OUTPUT_READY], t[:, :, END])[sel]
+        waves = np.where(waves > 0, waves, t[:, :, COMPUTE_DONE][sel])
+        print(f"  {NAMES[op]:10s} {st.min():7.2f} | {q(dep, (10, 50, 100))} | {q(waves, (50, 100))} | {q(sig, (50, 100))} | "
+              f"{q(done, (50, 100))}")
     sel = ins[:, :, 0] == 7
     if sel.any():
-        print(f"  {'lm-head':10s} {t[:, :, 0][sel].min():7.2f} | {np.percentile(t[:, :, 1][sel], 50):7.2f} (p50) | "
-              f"{t[:, :, 4][sel].max():7.2f} (max)")
+        print(f"  {'lm-head':10s} {t[:, :, START][sel].min():7.2f} | {np.percentile(t[:, :, DEP_READY][sel], 50):7.2f} (p50) | "
+              f"{t[:, :, END][sel].max():7.2f} (max)")
+    # per layer period: from one layer's QKV dependency (median worker) to the next one's
+    deps = [np.percentile(t[:, :, DEP_READY][(ins[:, :, 0] == 1) & (ins[:, :, 1] == l)], 50) for l in range(opts["layers"])]
+    if len(deps) > 2:
+        print(f"\nlayer period (QKV dependency seen, median worker, layer to layer): mean {np.mean(np.diff(deps[1:])):.2f} us")
 
 
 if __name__ == "__main__":

@@ -247,13 +247,45 @@ def test_timings_are_recorded_on_request():
     t = g.timings.cpu()
     ins = g.instructions.cpu()
     real = ins[:, :, 0] != 0
-    assert torch.equal(t[:, :, 5][real], ins[:, :, 0][real])            # opcode echoed
+    from megakernels_amd.scripts import timeline as tl
+
+    assert torch.equal(t[:, :, tl.OPCODE][real], ins[:, :, 0][real])    # opcode echoed
     # the records are the low 32 bits of one device-wide clock: start <= dependency seen <= input
     # ready <= rows done <= end for every instruction, and nothing took longer than a second
-    ticks = t[:, :, :5].to(torch.int64)
-    for earlier, later in ((0, 1), (1, 2), (2, 3), (3, 4)):
-        gap = (ticks[:, :, later] - ticks[:, :, earlier])[real] % (1 << 32)
+    ticks = t.to(torch.int64)
+
+    def ordered(earlier, later, where):
+        gap = (ticks[:, :, later] - ticks[:, :, earlier])[where] % (1 << 32)
         assert bool((gap < 100_000_000).all()), (earlier, later)
+
+    for earlier, later in ((0, 1), (1, 2), (2, 3), (3, 4)):
+        ordered(earlier, later, real)
+    # the waves that do the work stamp the reference's own event slots (include/util.cuh:215-246):
+    # measured, in order, for every matvec instruction that had rows
+    matvec = real & (ins[:, :, 0] != 2) & (ins[:, :, 0] != 3) & (t[:, :, tl.FIRST_USE] != 0)
+    assert int(matvec.sum()) > 0
+    chain = (tl.START, tl.AT_GMEM_WAIT, tl.DONE_GMEM_WAIT, tl.LAUNCHER_START, tl.FIRST_USE, tl.LAST_USE,
+             tl.AT_GMEM_STORE, tl.END)
+    for earlier, later in zip(chain, chain[1:]):
+        ordered(earlier, later, matvec)
+    ordered(tl.FIRST_LOAD, tl.LAST_LOAD, matvec)
+    ordered(tl.LAST_LOAD, tl.LAST_USE, matvec)
+    signalling = matvec & (ins[:, :, 0] != 7)   # the LM head signals nobody inside the launch
+    for earlier, later in ((tl.AT_GMEM_STORE, tl.DONE_GMEM_STORE), (tl.DONE_GMEM_STORE, tl.OUTPUT_READY),
+                           (tl.OUTPUT_READY, tl.END)):
+        ordered(earlier, later, signalling)
+    assert torch.equal(t[:, :, tl.DONE_GMEM_WAIT][matvec], t[:, :, tl.DEP_READY][matvec])
+    # attention and merge: the working waves stamp first use, stores and signal
+    for op in (2, 3):
+        sel = real & (ins[:, :, 0] == op)
+        if int(sel.sum()):
+            for earlier, later in ((tl.START, tl.AT_GMEM_STORE), (tl.AT_GMEM_STORE, tl.DONE_GMEM_STORE),
+                                   (tl.DONE_GMEM_STORE, tl.OUTPUT_READY)):
+                ordered(earlier, later, sel)
+            # (in attention the storing waves signal on their own, after the controller wave has moved
+            # on: its END can precede OUTPUT_READY; a merge leaves together, after the signal)
+            if op == 3:
+                ordered(tl.OUTPUT_READY, tl.END, sel)
     # one clock for all workers: the whole launch spans well under a second
     starts = ticks[:, :, 0][real]
     assert int(((starts - starts.min()) % (1 << 32)).max()) < 100_000_000

@@ -324,24 +324,40 @@ def test_repl_conversation_on_the_pytorch_generator(tmp_path):
 
 
 def test_timing_records_in_the_reference_event_slots():
-    """scripts/timeline.reference_event_layout: the kernel's five stamps per instruction (low 32 bits
-    of one device clock) re-laid into the reference's event slots (include/util.cuh:215-246), as ticks
-    since the first instruction started - also across a wrap of the 32-bit clock."""
-    from megakernels_amd.scripts.timeline import REFERENCE_EVENTS, reference_event_layout
+    """scripts/timeline.reference_event_layout: the kernel stamps the reference's event slots
+    (include/util.cuh:215-246) itself, with the low 32 bits of one device clock; the re-laid record holds
+    the same events as ticks since the first instruction started - also across a wrap of the 32-bit
+    clock - with the stages only the reference has (slots 1-3) set to the start, unstamped slots zero."""
+    from megakernels_amd.scripts import timeline as tl
 
     ins = torch.zeros(2, 3, 32, dtype=torch.int32)
     ins[0, 0, 0], ins[0, 1, 0], ins[1, 0, 0] = 1, 6, 2          # worker 1 has two NoOps
     raw = torch.zeros(2, 3, 128, dtype=torch.int64)
     base = (1 << 32) - 50                                         # the clock wraps during the launch
-    raw[0, 0, :6] = torch.tensor([base + 0, base + 10, base + 20, base + 70, base + 90, 1])
-    raw[0, 1, :6] = torch.tensor([base + 100, base + 100, base + 130, base + 400, base + 420, 6])
-    raw[1, 0, :6] = torch.tensor([base + 5, base + 40, base + 45, base + 300, base + 310, 2])
+
+    def record(w, s, opcode, **at):
+        raw[w, s, tl.OPCODE] = opcode
+        for name, tick in at.items():
+            raw[w, s, getattr(tl, name)] = base + tick
+
+    record(0, 0, 1, START=0, DEP_READY=10, DONE_GMEM_WAIT=10, INPUT_READY=20, LAUNCHER_START=20, COMPUTE_DONE=70,
+           AT_GMEM_STORE=75, DONE_GMEM_STORE=85, OUTPUT_READY=88, END=90, FIRST_LOAD=2, FIRST_USE=21, LAST_USE=66)
+    raw[0, 0, tl.CONSUMER_START + 2 * 3] = base + 22               # consumer wave 3: first row ...
+    raw[0, 0, tl.CONSUMER_START + 2 * 3 + 1] = base + 69           # ... and last row done
+    record(0, 1, 6, START=100, DEP_READY=100, INPUT_READY=130, COMPUTE_DONE=400, DONE_GMEM_STORE=415, END=420)
+    record(1, 0, 2, START=5, DEP_READY=40, INPUT_READY=45, COMPUTE_DONE=300, OUTPUT_READY=309, END=310)
     timings = (raw & 0xFFFFFFFF).to(torch.int32)                 # what the kernel stores
-    out = reference_event_layout(timings, ins)
+    out = tl.reference_event_layout(timings, ins)
     assert out.shape == timings.shape and out.dtype == torch.int32
-    assert out[0, 0, 0] == 0 and out[0, 0, 4] == 90 and out[0, 0, 45] == 10 and out[0, 0, 11] == 20 and out[0, 0, 46] == 70
-    assert out[0, 1, 0] == 100 and out[0, 1, 47] == 420 and out[1, 0, 0] == 5 and out[1, 0, 54] == 310
+    assert out[0, 0, 0] == 0 and out[0, 0, 4] == 90 and out[0, 0, 45] == 10 and out[0, 0, 7] == 20 and out[0, 0, 46] == 75
+    assert out[0, 0, 47] == 85 and out[0, 0, 54] == 88 and out[0, 0, 48] == 2 and out[0, 0, 49] == 21 and out[0, 0, 52] == 66
+    assert out[0, 0, 11 + 6] == 22 and out[0, 0, 11 + 7] == 69 and out[0, 0, 11] == 0     # wave 0 had no row
+    assert out[0, 1, 0] == 100 and out[0, 1, 47] == 415 and out[0, 1, 46] == 0 and out[1, 0, 0] == 5 and out[1, 0, 54] == 309
+    # the reference's fetch / page / semaphore stages: over when the instruction starts
+    assert [int(out[0, 1, k]) for k in (1, 2, 3)] == [100, 100, 100] and int(out[1, 0, 2]) == 5
+    assert int(out[0, 0, tl.OPCODE]) == 1 and int(out[1, 0, tl.OPCODE]) == 2
     assert int(out[1, 1:].abs().sum()) == 0 and int(out[0, 2].abs().sum()) == 0
-    unused = [i for i in range(128) if i not in REFERENCE_EVENTS]
+    unused = [i for i in range(128) if i not in tl.TIME_SLOTS and i not in tl.REFERENCE_ONLY_STAGES and i != tl.OPCODE]
     assert int(out[:, :, unused].abs().sum()) == 0
-    assert REFERENCE_EVENTS[0] == 0 and REFERENCE_EVENTS[4] == 4   # controller start / end coincide with the kernel's own
+    t, stamped = tl.microseconds(timings.numpy())
+    assert abs(t[0, 1, tl.END] - 4.2) < 1e-9 and bool(stamped[0, 0, tl.FIRST_USE]) and not bool(stamped[0, 1, tl.FIRST_USE])
