@@ -874,7 +874,10 @@ __device__ __forceinline__ bool matvec_batch(const Ctx &c, int ntasks, bool need
 
 // malformed instruction: every wave evaluates the same condition and leaves; the controller records it
 __device__ __forceinline__ bool bail(const Ctx &c, int code, int *refusal) {
-    if (c.controller && c.lane == 0) record_status(c, code);
+    if (c.controller && c.lane == 0) {
+        record_status(c, code);
+        c.sm->abort = code;
+    }
     *refusal = code;
     return false;
 }
@@ -915,7 +918,7 @@ __host__ __device__ constexpr bool joint_groups(uint32_t flags, int G, int in_di
 
 // Decodes the matvec instruction in queue slot `slot` (executed once per launch by one thread per
 // slot; the launch arguments come from the kernel's argument registers).
-__device__ __forceinline__ void decode_matvec(SmemPtr sm, int slot, const mk_llama_args &a) {
+__device__ __forceinline__ void decode_matvec(SmemPtr sm, int slot, ArgsRef a) {
     const InsPtr ins = sm->queue[slot];
     const int hid = a.hidden_size, inter = a.intermediate_size;
     const int opcode = ins[0], layer = ins[1];
@@ -2173,6 +2176,196 @@ static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot
 // ---------------------------------------------------------------------------------------------
 // the persistent kernel
 // ---------------------------------------------------------------------------------------------
+// Everything the instruction loop needs between two instructions lives in LDS (the launch arguments,
+// the queue window, the abort flag): the loop itself keeps a handful of values in registers, nothing
+// in scratch memory, so that a handler's return is not followed by a reload from memory - which
+// would be a round trip through the vector memory path on the way to every next instruction.
+
+// Instruction fetch (reference: controller warp, include/controller/instruction_fetch.cuh:10-27):
+// a window of the worker's queue is copied into LDS and its matvec instructions are decoded, so that
+// taking an instruction never waits on HBM.  The usual queue fits the window and is fetched once per
+// launch; a longer one goes through window by window, every step.
+static __device__ __noinline__ void fetch_window(SmemPtr sm, int base) {
+    ArgsRef a = sm->args;
+    const int tid = (int)threadIdx.x;
+    const int count = min(kQueueSlots, a.num_slots - base);
+    const MK_GLOBAL int *queue = as_global(a.instructions) + ((size_t)blockIdx.x * a.num_slots + base) * MK_INSTRUCTION_WORDS;
+    MK_LDS int *dst = &sm->queue[0][0];
+    for (int i = tid; i < count * MK_INSTRUCTION_WORDS; i += kThreads) dst[i] = queue[i];
+    if (tid == 0) {
+        sm->window_base = base;
+        sm->window_count = count;
+        sm->parked_slot = -1;
+    }
+    wg_barrier();
+    for (int slot = tid; slot < count; slot += kThreads) {
+        const int opcode = sm->queue[slot][0];
+        if (opcode == 1 || (opcode >= 4 && opcode <= 6)) decode_matvec(sm, slot, a);
+    }
+    wg_barrier();
+}
+
+// End of a step.  The last workgroup to get here folds the sharded counters into `barriers` (or
+// zeroes `barriers`), leaves the shards zeroed, and turns the workers' LM-head maxima into the step's
+// token.  With more steps to go it then publishes the step, and everybody else waits for that before
+// starting on the next token.  Returns whether another step follows.
+template <bool TR>
+static __device__ __noinline__ bool end_of_step(SmemPtr sm, int step, int steps) {
+    ArgsRef a = sm->args;
+    const int tid = (int)threadIdx.x;
+    const WsLayout wl = ws_layout(a.num_layers, a.hidden_size, a.intermediate_size, a.matvec_reduction_size);
+    int *status = static_cast<int *>(a.workspace) + wl.status;
+    wait_stores();
+    wg_barrier();
+    if (tid == 0) {
+        const int done = __hip_atomic_fetch_add(as_global(&status[kDoneSlot]), 1, __ATOMIC_RELAXED, AG);
+        sm->last_flag = done == (int)gridDim.x * (step + 1) - 1;
+    }
+    wg_barrier();
+    const bool more = step + 1 < steps && sm->abort == 0;
+    if (sm->last_flag) {
+        // One thread per (counter, shard), two pairs per trip with both loads in flight, and the
+        // workers' maxima requested before the fold: the step's token waits for one round trip
+        // here, not for a chain of them.
+        const int counters = a.num_layers * kHotRows;
+        int *shards = static_cast<int *>(a.workspace) + wl.shards;
+        const int cols = a.num_attention_heads + 2 * a.num_kv_heads;
+        const bool reset = (a.flags & MK_FLAG_RESET_BARRIERS) != 0;
+        int *maxima = static_cast<int *>(a.workspace) + wl.argmax;
+        int *barriers = a.barriers;
+        constexpr int kMaxTrips = (kMaxWorkers + kThreads - 1) / kThreads;
+        uint64_t reported[kMaxTrips];
+#pragma unroll
+        for (int k = 0; k < kMaxTrips; k++) {
+            const int w = tid + k * kThreads;
+            reported[k] = a.token_out && w < (int)gridDim.x ? ld_u64(maxima + 2 * w) : 0;
+        }
+        // k = (replica, shard, counter); every copy is zeroed, the first one is what gets counted
+        auto shard_at = [&](int k) { return shards + k; };
+        auto fold = [&](int k, int v) {
+            if (v == 0) return;
+            st_i32(shard_at(k), 0);
+            const int i = k % counters;
+            if (!reset && k < counters * kShards) add_i32(barriers + ((size_t)(i / kHotRows) * MK_BARRIER_ROWS + 2 + i % kHotRows) * cols, v);
+        };
+        const int pairs = counters * kShards * kReplicas;
+        for (int k = tid; k < pairs; k += 2 * kThreads) {
+            const int k2 = k + kThreads;
+            const int v = ld_i32(shard_at(k));
+            const int v2 = k2 < pairs ? ld_i32(shard_at(k2)) : 0;
+            fold(k, v);
+            if (k2 < pairs) fold(k2, v2);
+        }
+        {
+            // the padded per-head counters, four looks in flight per thread and trip
+            int *pads = static_cast<int *>(a.workspace) + wl.pads;
+            const int pc = pad_cols(a.hidden_size), npad = a.num_layers * 2 * pc;
+            for (int k0 = tid; k0 < npad; k0 += 4 * kThreads) {
+                int v[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int k = k0 + u * kThreads;
+                    v[u] = k < npad ? ld_i32(pads + (size_t)k * kPadInts) : 0;
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int k = k0 + u * kThreads;
+                    if (v[u] == 0) continue;
+                    st_i32(pads + (size_t)k * kPadInts, 0);
+                    const int col = k % pc, lr = k / pc;
+                    if (!reset && col < cols)
+                        add_i32(barriers + ((size_t)(lr / 2) * MK_BARRIER_ROWS + lr % 2) * cols + col, v[u]);
+                }
+            }
+        }
+        if (reset) {
+            const int words = a.num_layers * MK_BARRIER_ROWS * cols;
+            for (int i = tid; i < words; i += kThreads) st_i32(barriers + i, 0);
+        }
+        if (a.token_out) {
+            // the workers' LM-head maxima -> the step's token
+            float v = -INFINITY;
+            int idx = INT_MAX;
+#pragma unroll
+            for (int k = 0; k < kMaxTrips; k++) {
+                const int stored = (int)(reported[k] >> 32);
+                if (stored) {
+                    const float wv = __builtin_bit_cast(float, (int)(uint32_t)reported[k]);
+                    if (wv > v || (wv == v && stored - 1 < idx)) {
+                        v = wv;
+                        idx = stored - 1;
+                    }
+                    st_i32(maxima + 2 * (tid + k * kThreads) + 1, 0);
+                }
+            }
+            argmax_combine_wave(v, idx);
+            if (tid % 64 == 0) {
+                sm->out[2 * (tid / 64)] = v;
+                sm->flags[tid / 64] = idx;
+            }
+            wg_barrier();
+            if (tid == 0) {
+                for (int w = 1; w < kThreads / 64; w++) {
+                    const float wv = sm->out[2 * w];
+                    const int wi = sm->flags[w];
+                    if (wv > v || (wv == v && wi < idx)) {
+                        v = wv;
+                        idx = wi;
+                    }
+                }
+                const int token = idx == INT_MAX ? 0 : idx;
+                st_u64(a.token_out + step, (uint64_t)token);
+                sm->token = token;
+            }
+        }
+        if (tid == 0) st_i32(&status[kEpochSlot], (int)(sm->k.epoch + 1u));
+        if (more) {
+            // everything the next step relies on (zeroed counters, the token) has landed before
+            // the step is published
+            wait_stores();
+            wg_barrier();
+            if (tid == 0) st_i32(&status[kStepSlot], step + 1);
+        } else if (tid == 0) {
+            st_i32(&status[kDoneSlot], 0);
+            st_i32(&status[kStepSlot], 0);
+        }
+    } else if (more && tid < 64) {
+        // one wave watches for the step's publication (and for a failure anywhere)
+        const long long t0 = wall_clock64();
+        const long long limit = (long long)(a.spin_limit_us ? a.spin_limit_us : 2000000u) * 100;
+        bool ok = true;
+        while (true) {
+            const int published = ld_i32(&status[kStepSlot]);
+            const int failure = ld_i32(&status[0]);
+            if (failure != 0) {
+                ok = false;
+                break;
+            }
+            if (published > step) break;
+            if (wall_clock64() - t0 > limit) {
+                if (tid == 0) record_status(make_ctx<TR>(sm, 0, 0), MK_STATUS_BARRIER_TIMEOUT);
+                ok = false;
+                break;
+            }
+            __builtin_amdgcn_s_sleep(MK_POLL_SLEEP);
+        }
+        compiler_fence();
+        const uint64_t token = ok ? ld_u64(a.token_out + step) : 0;
+        if (tid == 0) {
+            if (ok) sm->token = (int)token;
+            else sm->abort = 1;
+        }
+    }
+    if (!more) return false;
+    if (tid == 0) {
+        sm->args.pos_id = a.pos_id + 1;
+        sm->k.epoch += 1u;
+        sm->parked_slot = -1;
+    }
+    wg_barrier();
+    return sm->abort == 0;
+}
+
 template <int KC_HID, int KC_RED, int D, bool TR>
 __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args a) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -2215,254 +2408,91 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
         sm->k.down_jobs = (a.intermediate_size / a.matvec_reduction_size) * (a.hidden_size / 16);
         sm->k.o_jobs = (a.hidden_size / a.matvec_reduction_size) * (a.hidden_size / 16);
     }
-    // Instruction fetch (reference: controller warp, include/controller/instruction_fetch.cuh:10-27):
-    // a window of the worker's queue is copied into LDS and its matvec instructions are decoded,
-    // so that taking an instruction never waits on HBM.  The usual queue fits the window and is
-    // fetched once per launch; a longer one goes through window by window, every step.
-    auto fetch_window = [&](int base) {
-        const int count = min(kQueueSlots, a.num_slots - base);
-        const int *queue = a.instructions + ((size_t)blockIdx.x * a.num_slots + base) * MK_INSTRUCTION_WORDS;
-        MK_LDS int *dst = &sm->queue[0][0];
-        for (int i = tid; i < count * MK_INSTRUCTION_WORDS; i += kThreads) dst[i] = queue[i];
-        if (tid == 0) {
-            sm->window_base = base;
-            sm->window_count = count;
-            sm->parked_slot = -1;
-        }
-        wg_barrier();
-        for (int slot = tid; slot < count; slot += kThreads) {
-            const int opcode = sm->queue[slot][0];
-            if (opcode == 1 || (opcode >= 4 && opcode <= 6)) decode_matvec(sm, slot, a);
-        }
-        wg_barrier();
-    };
-    fetch_window(0);
-
-    // The handlers get the address of a kernel-local word for their refusal code.  Besides carrying
-    // the code it keeps the calls from being marked as tail calls, which lets the compiler drop the
-    // callee-saved register traffic (dozens of scratch stores and reloads per instruction) from
-    // handlers that only this kernel calls.
-    int refusal = 0;
-    if (a.token_in && sm->token < 0) {
-        // every workgroup sees the same bad token and skips its queue
-        if (tid == kConsumerThreads) record_status(make_ctx<TR>(sm, 0, 0), MK_STATUS_BAD_TOKEN);
-        refusal = MK_STATUS_BAD_TOKEN;
-    }
     // A launch covers one decode step, or `num_steps` of them back to back: the token a step
     // produces starts the next one, at the next position.
     const int steps = a.num_steps > 1 ? a.num_steps : 1;
-    const WsLayout wl = ws_layout(a.num_layers, a.hidden_size, a.intermediate_size, a.matvec_reduction_size);
-    int *status = static_cast<int *>(a.workspace) + wl.status;
+    wg_barrier();  // the argument block and the token are in LDS
+    // a launch that was given a token outside the vocabulary: every workgroup sees the same bad token
+    // and skips its queue
+    const bool bad_token = a.token_in && uni(sm->token) < 0;
+    fetch_window(sm, 0);
+    if (bad_token && tid == kConsumerThreads) {
+        record_status(make_ctx<TR>(sm, 0, 0), MK_STATUS_BAD_TOKEN);
+        sm->abort = MK_STATUS_BAD_TOKEN;
+    }
+    // From here on nothing refers to the kernel's arguments: what the loop needs comes from LDS.
+    // The handlers get the address of a kernel-local word, into which a handler that refuses its
+    // instruction writes why.  Nothing reads the word on the way from one instruction to the next (the
+    // handlers' return values say whether to go on); it is there because a call that is handed the
+    // address of a local cannot be marked as a tail call, and only then does the compiler drop the
+    // callee-saved register traffic (dozens of scratch stores and reloads per instruction) from
+    // handlers that only this kernel calls.
+    int refusal = 0;
     for (int step = 0; step < steps; step++) {
-      for (int base = 0; base < a.num_slots && refusal == 0; base += kQueueSlots) {
-        if (sm->window_base != base) {
-            wg_barrier();  // nobody is still reading the window that goes
-            fetch_window(base);
-        }
-        const int window_slots = min(kQueueSlots, a.num_slots - base);
-        for (int slot = 0; slot < window_slots && refusal == 0; slot++) {
-            const int opcode = sm->queue[slot][0];
-            if (opcode == 0) continue;  // NoOp pads the queues (megakernels/scheduler.py:287-289)
-            {
-                const Ctx c = make_ctx<TR>(sm, slot, opcode);
-                trace_event(c, kEvStart);
-                if (c.trace && c.controller && c.lane == 0) st_plain_i32(c.trace + kEvOpcode, opcode);
+        bool stop = bad_token;
+        const int num_slots = uni(sm->args.num_slots);
+        for (int base = 0; base < num_slots && !stop; base += kQueueSlots) {
+            if (uni(sm->window_base) != base) {
+                wg_barrier();  // nobody is still reading the window that goes
+                fetch_window(sm, base);
             }
-            bool ok = true;
-            switch (opcode) {
-            case 1: ok = op_matvec<TR, 1, KC_HID>(sm, slot, &refusal); break;
-            case 2: ok = op_attention<TR, D>(sm, slot, &refusal); break;
-            case 3: ok = op_attention_reduction<TR, D>(sm, slot, &refusal); break;
-            case 4:
-                if constexpr (KC_HID == KC_RED && MK_PAIR_OPROJ_UPGATE) {
-                    if (slot + 1 < window_slots && sm->queue[slot + 1][0] == 5) {
-                        // rows can be parked when the wait is long (no attention just before, and a
-                        // partition merge between attention and O-proj: with a single partition per head
-                        // the wait is too short for it to pay) and the up/gate instruction is small
-                        // enough (two list entries: eight rows per wave)
-                        const bool park = MK_PARK_UPGATE && !a.skip_attn_reduction && (slot == 0 || sm->queue[slot - 1][0] != 2) &&
-                                          sm->queue[slot + 1][2] >= 0 && sm->queue[slot + 1][2] <= 2;
-                        const int executed = park ? op_oproj_upgate<TR, KC_HID, true>(sm, slot, &refusal)
-                                                  : op_oproj_upgate<TR, KC_HID, false>(sm, slot, &refusal);
-                        ok = executed > 0;
-                        slot += ok ? executed - 1 : 0;
-                        break;
-                    }
+            const int window_slots = min(kQueueSlots, num_slots - base);
+            for (int slot = 0; slot < window_slots; slot++) {
+                // (everything the loop branches on is the same in all lanes; saying so keeps the branches
+                // scalar and the loop's state in a few scalar registers)
+                const int opcode = uni(sm->queue[slot][0]);
+                if (opcode == 0) continue;  // NoOp pads the queues (megakernels/scheduler.py:287-289)
+                if constexpr (TR) {
+                    const Ctx c = make_ctx<TR>(sm, slot, opcode);
+                    trace_event(c, kEvStart);
+                    if (c.trace && c.controller && c.lane == 0) st_plain_i32(c.trace + kEvOpcode, opcode);
                 }
-                ok = op_matvec<TR, 4, KC_RED>(sm, slot, &refusal);
-                break;
-            case 5: ok = op_matvec<TR, 5, KC_HID>(sm, slot, &refusal); break;
-            case 6:
-            if constexpr (KC_HID == KC_RED && MK_PAIR_OPROJ_UPGATE && MK_PARK_UPGATE && MK_PARK_DOWN) {
-                if (sm->parked_slot == slot) {
-                    ok = op_matvec<TR, 6, KC_RED, 1>(sm, slot, &refusal);
-                    break;
-                }
-            }
-            ok = op_matvec<TR, 6, KC_RED>(sm, slot, &refusal);
-            break;
-            case 7: ok = op_lm_head<TR, KC_HID>(sm, slot, &refusal); break;
-            default: ok = bail(make_ctx<TR>(sm, slot, opcode), MK_STATUS_BAD_OPCODE, &refusal);  // reference: trap, include/util.cuh:38
-            }
-            if (!ok) break;
-            trace_event(make_ctx<TR>(sm, slot, sm->queue[slot][0]), kEvEnd);
-        }
-        if (sm->abort) break;
-      }
-        if (refusal && tid == 0) sm->abort = refusal;
-
-        // End of a step.  The last workgroup to get here folds the sharded counters into `barriers`
-        // (or zeroes `barriers`), leaves the shards zeroed, and turns the workers' LM-head maxima into
-        // the step's token.  With more steps to go it then publishes the step, and everybody else
-        // waits for that before starting on the next token.
-        wait_stores();
-        wg_barrier();
-        if (tid == 0) {
-            const int done = __hip_atomic_fetch_add(&status[kDoneSlot], 1, __ATOMIC_RELAXED, AG);
-            sm->last_flag = done == (int)gridDim.x * (step + 1) - 1;
-        }
-        wg_barrier();
-        const bool more = step + 1 < steps && sm->abort == 0;
-        if (sm->last_flag) {
-            // One thread per (counter, shard), two pairs per trip with both loads in flight, and the
-            // workers' maxima requested before the fold: the step's token waits for one round trip
-            // here, not for a chain of them.
-            const int counters = a.num_layers * kHotRows;
-            int *shards = static_cast<int *>(a.workspace) + wl.shards;
-            const int cols = a.num_attention_heads + 2 * a.num_kv_heads;
-            const bool reset = (a.flags & MK_FLAG_RESET_BARRIERS) != 0;
-            int *maxima = static_cast<int *>(a.workspace) + wl.argmax;
-            constexpr int kMaxTrips = (kMaxWorkers + kThreads - 1) / kThreads;
-            uint64_t reported[kMaxTrips];
-#pragma unroll
-            for (int k = 0; k < kMaxTrips; k++) {
-                const int w = tid + k * kThreads;
-                reported[k] = a.token_out && w < (int)gridDim.x ? ld_u64(maxima + 2 * w) : 0;
-            }
-            // k = (replica, shard, counter); every copy is zeroed, the first one is what gets counted
-            auto shard_at = [&](int k) { return shards + k; };
-            auto fold = [&](int k, int v) {
-                if (v == 0) return;
-                st_i32(shard_at(k), 0);
-                const int i = k % counters;
-                if (!reset && k < counters * kShards) add_i32(a.barriers + ((size_t)(i / kHotRows) * MK_BARRIER_ROWS + 2 + i % kHotRows) * cols, v);
-            };
-            const int pairs = counters * kShards * kReplicas;
-            for (int k = tid; k < pairs; k += 2 * kThreads) {
-                const int k2 = k + kThreads;
-                const int v = ld_i32(shard_at(k));
-                const int v2 = k2 < pairs ? ld_i32(shard_at(k2)) : 0;
-                fold(k, v);
-                if (k2 < pairs) fold(k2, v2);
-            }
-            {
-                // the padded per-head counters, four looks in flight per thread and trip
-                int *pads = static_cast<int *>(a.workspace) + wl.pads;
-                const int pc = pad_cols(a.hidden_size), npad = a.num_layers * 2 * pc;
-                for (int k0 = tid; k0 < npad; k0 += 4 * kThreads) {
-                    int v[4];
-#pragma unroll
-                    for (int u = 0; u < 4; u++) {
-                        const int k = k0 + u * kThreads;
-                        v[u] = k < npad ? ld_i32(pads + (size_t)k * kPadInts) : 0;
-                    }
-#pragma unroll
-                    for (int u = 0; u < 4; u++) {
-                        const int k = k0 + u * kThreads;
-                        if (v[u] == 0) continue;
-                        st_i32(pads + (size_t)k * kPadInts, 0);
-                        const int col = k % pc, lr = k / pc;
-                        if (!reset && col < cols)
-                            add_i32(a.barriers + ((size_t)(lr / 2) * MK_BARRIER_ROWS + lr % 2) * cols + col, v[u]);
-                    }
-                }
-            }
-            if (reset) {
-                const int words = a.num_layers * MK_BARRIER_ROWS * cols;
-                for (int i = tid; i < words; i += kThreads) st_i32(a.barriers + i, 0);
-            }
-            if (a.token_out) {
-                // the workers' LM-head maxima -> the step's token
-                float v = -INFINITY;
-                int idx = INT_MAX;
-#pragma unroll
-                for (int k = 0; k < kMaxTrips; k++) {
-                    const int stored = (int)(reported[k] >> 32);
-                    if (stored) {
-                        const float wv = __builtin_bit_cast(float, (int)(uint32_t)reported[k]);
-                        if (wv > v || (wv == v && stored - 1 < idx)) {
-                            v = wv;
-                            idx = stored - 1;
-                        }
-                        st_i32(maxima + 2 * (tid + k * kThreads) + 1, 0);
-                    }
-                }
-                argmax_combine_wave(v, idx);
-                if (tid % 64 == 0) {
-                    sm->out[2 * (tid / 64)] = v;
-                    sm->flags[tid / 64] = idx;
-                }
-                wg_barrier();
-                if (tid == 0) {
-                    for (int w = 1; w < kThreads / 64; w++) {
-                        const float wv = sm->out[2 * w];
-                        const int wi = sm->flags[w];
-                        if (wv > v || (wv == v && wi < idx)) {
-                            v = wv;
-                            idx = wi;
+                bool ok = true;
+                switch (opcode) {
+                case 1: ok = uni((int)op_matvec<TR, 1, KC_HID>(sm, slot, &refusal)) != 0; break;
+                case 2: ok = uni((int)op_attention<TR, D>(sm, slot, &refusal)) != 0; break;
+                case 3: ok = uni((int)op_attention_reduction<TR, D>(sm, slot, &refusal)) != 0; break;
+                case 4:
+                    if constexpr (KC_HID == KC_RED && MK_PAIR_OPROJ_UPGATE) {
+                        if (slot + 1 < window_slots && uni(sm->queue[slot + 1][0]) == 5) {
+                            // rows can be parked when the wait is long (no attention just before, and a
+                            // partition merge between attention and O-proj: with a single partition per head
+                            // the wait is too short for it to pay) and the up/gate instruction is small
+                            // enough (two list entries: eight rows per wave)
+                            const int entries = uni(sm->queue[slot + 1][2]);
+                            const bool park = MK_PARK_UPGATE && !uni(sm->args.skip_attn_reduction) &&
+                                              (slot == 0 || uni(sm->queue[slot - 1][0]) != 2) && entries >= 0 && entries <= 2;
+                            const int executed = uni(park ? op_oproj_upgate<TR, KC_HID, true>(sm, slot, &refusal)
+                                                          : op_oproj_upgate<TR, KC_HID, false>(sm, slot, &refusal));
+                            ok = executed > 0;
+                            slot += ok ? executed - 1 : 0;
+                            break;
                         }
                     }
-                    const int token = idx == INT_MAX ? 0 : idx;
-                    st_u64(a.token_out + step, (uint64_t)token);
-                    sm->token = token;
+                    ok = uni((int)op_matvec<TR, 4, KC_RED>(sm, slot, &refusal)) != 0;
+                    break;
+                case 5: ok = uni((int)op_matvec<TR, 5, KC_HID>(sm, slot, &refusal)) != 0; break;
+                case 6:
+                    if constexpr (KC_HID == KC_RED && MK_PAIR_OPROJ_UPGATE && MK_PARK_UPGATE && MK_PARK_DOWN) {
+                        if (uni(sm->parked_slot) == slot) {
+                            ok = uni((int)op_matvec<TR, 6, KC_RED, 1>(sm, slot, &refusal)) != 0;
+                            break;
+                        }
+                    }
+                    ok = uni((int)op_matvec<TR, 6, KC_RED>(sm, slot, &refusal)) != 0;
+                    break;
+                case 7: ok = uni((int)op_lm_head<TR, KC_HID>(sm, slot, &refusal)) != 0; break;
+                default: ok = bail(make_ctx<TR>(sm, slot, opcode), MK_STATUS_BAD_OPCODE, &refusal);  // reference: trap, include/util.cuh:38
                 }
-            }
-            if (tid == 0) st_i32(&status[kEpochSlot], (int)(sm->k.epoch + 1u));
-            if (more) {
-                // everything the next step relies on (zeroed counters, the token) has landed before
-                // the step is published
-                wait_stores();
-                wg_barrier();
-                if (tid == 0) st_i32(&status[kStepSlot], step + 1);
-            } else if (tid == 0) {
-                st_i32(&status[kDoneSlot], 0);
-                st_i32(&status[kStepSlot], 0);
-            }
-        } else if (more && tid < 64) {
-            // one wave watches for the step's publication (and for a failure anywhere)
-            const long long t0 = wall_clock64();
-            const long long limit = (long long)(a.spin_limit_us ? a.spin_limit_us : 2000000u) * 100;
-            bool ok = true;
-            while (true) {
-                const int published = ld_i32(&status[kStepSlot]);
-                const int failure = ld_i32(&status[0]);
-                if (failure != 0) {
-                    ok = false;
+                if (!ok) {
+                    stop = true;
                     break;
                 }
-                if (published > step) break;
-                if (wall_clock64() - t0 > limit) {
-                    if (tid == 0) record_status(make_ctx<TR>(sm, 0, 0), MK_STATUS_BARRIER_TIMEOUT);
-                    ok = false;
-                    break;
-                }
-                __builtin_amdgcn_s_sleep(MK_POLL_SLEEP);
-            }
-            compiler_fence();
-            const uint64_t token = ok ? ld_u64(a.token_out + step) : 0;
-            if (tid == 0) {
-                if (ok) sm->token = (int)token;
-                else sm->abort = 1;
+                if constexpr (TR) trace_event(make_ctx<TR>(sm, slot, sm->queue[slot][0]), kEvEnd);
             }
         }
-        if (!more) break;
-        if (tid == 0) {
-            sm->args.pos_id = a.pos_id + step + 1;
-            sm->k.epoch += 1u;
-            sm->parked_slot = -1;
-        }
-        wg_barrier();
-        if (sm->abort) break;
+        if (stop && refusal != 0 && tid == 0) sm->abort = refusal;
+        if (!uni((int)end_of_step<TR>(sm, step, steps))) break;
     }
 }
 
