@@ -1487,15 +1487,23 @@ template <> struct FirstBuffers<4> { typedef BufMap<0, 1, 2, 3> type; };
 template <> struct FirstBuffers<5> { typedef BufMap<0, 1, 2, 3, 4> type; };
 template <> struct FirstBuffers<6> { typedef BufMap<0, 1, 2, 3, 4, 5> type; };
 
+// The two sides of an instruction.  The controller wave runs its side inlined into the kernel's
+// instruction loop: leaving a function with the signal's atomics still on their way would mean
+// waiting for them (calls and returns wait for all outstanding memory operations), which is a round
+// trip through memory between an instruction's signal and the first look at the next one's
+// dependency - on the worker that signals last, the round trip the next phase waits for.  The
+// consumer waves, which own the big register allocations, call one function per instruction kind.
+enum { kConsumerRole = 0, kControllerRole = 1 };
+
 // One matvec instruction (opcode OP, row width KC chunks).
-template <bool TR, int OP, int KC, int PARKED = 0>
-static __device__ __noinline__ bool op_matvec(SmemPtr lds, int slot, int *refusal) {
+template <bool TR, int OP, int KC, int PARKED, int ROLE>
+__device__ __forceinline__ bool matvec_impl(SmemPtr lds, int slot, int *refusal) {
     constexpr int PF = rows_in_flight<KC>(pf_of(OP));
     typedef typename FirstBuffers<PF>::type Map;
     const Ctx c = make_ctx<TR>(lds, slot, OP);
     MatvecDesc d;
     if (!describe_matvec(lds, slot, OP, d)) return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
-    if (c.controller) return control_matvec<KC>(c);
+    if constexpr (ROLE == kControllerRole) return control_matvec<KC>(c);
     const int mine = rows_of_wave(d.ntasks, c.wave);
     uint4 pool[PF][KC];
     wg_barrier();  // entry: the controller's first requests are out
@@ -1503,6 +1511,10 @@ static __device__ __noinline__ bool op_matvec(SmemPtr lds, int slot, int *refusa
     request_rows<KC, Map>(c, pool, d, 0, mine > PARKED ? mine - PARKED : 0);
     const bool ok = consumer_run<KC, Map, PF, PARKED>(c, pool, d, mine, (MK_LDS const unsigned char *)lds->park + c.wave * (KC * 1024));
     return ok;
+}
+template <bool TR, int OP, int KC, int PARKED = 0>
+static __device__ __noinline__ bool op_matvec(SmemPtr lds, int slot, int *refusal) {
+    return matvec_impl<TR, OP, KC, PARKED, kConsumerRole>(lds, slot, refusal);
 }
 
 // O-proj followed directly by up/gate, as one handler.  O-proj is short (two rows per wave in the
@@ -1531,14 +1543,7 @@ static __device__ __noinline__ int op_oproj_upgate(SmemPtr lds, int slot, int *r
         return 0;
     }
     const bool pair = describe_matvec(lds, slot + 1, 5, dsu);
-    if (co.controller) {
-        if (!control_matvec<KC>(co)) return 0;
-        if (!pair) return 1;
-        trace_event(co, kEvEnd);
-        trace_event(cu, kEvStart);
-        if (cu.trace && cu.lane == 0) st_plain_i32(cu.trace + kEvOpcode, 5);
-        return control_matvec<KC>(cu) ? 2 : 0;
-    }
+    // (consumer waves only: the controller wave takes the two instructions one after the other)
     if (!pair) dsu = dso;  // never fetched: the requests below become no-ops
     const int mine_o = rows_of_wave(dso.ntasks, co.wave);
     const int mine_u = pair ? rows_of_wave(dsu.ntasks, co.wave) : 0;
@@ -1732,8 +1737,8 @@ __device__ __forceinline__ MergedPair merge_partitions(const Ctx &c, int head, i
 // tokens in increasing order and slots are combined by a pairwise tree (token groups of a wave,
 // then waves).  A token's row is spread over D/8 lanes, 8 dims each.
 // ---------------------------------------------------------------------------------------------
-template <bool TR, int D>
-static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *refusal) {
+template <bool TR, int D, int ROLE>
+__device__ __forceinline__ bool attention_impl(SmemPtr lds, int slot, int *refusal) {
     const InsPtr ins = lds->queue[slot];
     const Ctx c = make_ctx<TR>(lds, slot, ins[0]);
     constexpr int LPT = D / 8;                   // lanes per token
@@ -1761,7 +1766,7 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
     const int h0 = kvh * G;
     const int rounds = (T + NSLOT - 1) / NSLOT;
 
-    if (c.controller) {
+    if constexpr (ROLE == kControllerRole) {
         // wait: Q heads, K head and V head of this step are complete (python_vm.py:281-290)
         const int col = c.lane < G ? h0 + c.lane : c.lane == G ? H + kvh : H + KVH + kvh;
         const bool mine = c.lane < G + 2;
@@ -2100,13 +2105,17 @@ static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *ref
     }
     return true;
 }
+template <bool TR, int D>
+static __device__ __noinline__ bool op_attention(SmemPtr lds, int slot, int *refusal) {
+    return attention_impl<TR, D, kConsumerRole>(lds, slot, refusal);
+}
 
 // ---------------------------------------------------------------------------------------------
 // opcode 3: log-sum-exp merge of attention partitions  (python_vm.py:349-393;
 // reference device op: demos/low-latency-llama/attention_reduction.cu:18-339)
 // ---------------------------------------------------------------------------------------------
-template <bool TR, int D>
-static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot, int *refusal) {
+template <bool TR, int D, int ROLE>
+__device__ __forceinline__ bool reduction_impl(SmemPtr lds, int slot, int *refusal) {
     const InsPtr ins = lds->queue[slot];
     const Ctx c = make_ctx<TR>(lds, slot, ins[0]);
     ArgsRef a = c.sm->args;
@@ -2128,7 +2137,7 @@ static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot
     // the counters do not queue behind bulk loads of its own.)  Everybody leaves together, after the
     // signal: the next instruction starts with bulk weight requests, and a CU serves its requests in
     // order.
-    if (c.tid < R * TPH) {
+    if (ROLE == kConsumerRole && c.tid < R * TPH) {
         const int h = c.tid / TPH, j = c.tid % TPH, d = j * 2;
         const int head = hs + h;
         const bool leader = j == 0;
@@ -2171,6 +2180,25 @@ static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot
     trace_event(c, kEvInputReady);
     trace_event(c, kEvComputeDone);
     return c.sm->abort == 0;
+}
+template <bool TR, int D>
+static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot, int *refusal) {
+    return reduction_impl<TR, D, kConsumerRole>(lds, slot, refusal);
+}
+
+// The controller wave's side of the instruction in `slot`.
+template <bool TR, int KC_HID, int KC_RED, int D>
+__device__ __forceinline__ bool controller_step(SmemPtr sm, int slot, int opcode, int *refusal) {
+    switch (opcode) {
+    case 1: return matvec_impl<TR, 1, KC_HID, 0, kControllerRole>(sm, slot, refusal);
+    case 2: return attention_impl<TR, D, kControllerRole>(sm, slot, refusal);
+    case 3: return reduction_impl<TR, D, kControllerRole>(sm, slot, refusal);
+    case 4: return matvec_impl<TR, 4, KC_RED, 0, kControllerRole>(sm, slot, refusal);
+    case 5: return matvec_impl<TR, 5, KC_HID, 0, kControllerRole>(sm, slot, refusal);
+    case 6: return matvec_impl<TR, 6, KC_RED, 0, kControllerRole>(sm, slot, refusal);
+    case 7: return op_lm_head<TR, KC_HID>(sm, slot, refusal);
+    default: return bail(make_ctx<TR>(sm, slot, opcode), MK_STATUS_BAD_OPCODE, refusal);  // reference: trap, include/util.cuh:38
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -2428,6 +2456,7 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
     // callee-saved register traffic (dozens of scratch stores and reloads per instruction) from
     // handlers that only this kernel calls.
     int refusal = 0;
+    const bool controller = uni(tid) >= kConsumerThreads;
     for (int step = 0; step < steps; step++) {
         bool stop = bad_token;
         const int num_slots = uni(sm->args.num_slots);
@@ -2448,7 +2477,9 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
                     if (c.trace && c.controller && c.lane == 0) st_plain_i32(c.trace + kEvOpcode, opcode);
                 }
                 bool ok = true;
-                switch (opcode) {
+                if (controller) {
+                    ok = uni((int)controller_step<TR, KC_HID, KC_RED, D>(sm, slot, opcode, &refusal)) != 0;
+                } else switch (opcode) {
                 case 1: ok = uni((int)op_matvec<TR, 1, KC_HID>(sm, slot, &refusal)) != 0; break;
                 case 2: ok = uni((int)op_attention<TR, D>(sm, slot, &refusal)) != 0; break;
                 case 3: ok = uni((int)op_attention_reduction<TR, D>(sm, slot, &refusal)) != 0; break;
