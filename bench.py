@@ -1,6 +1,6 @@
 """Headline benchmark: batch-1 greedy decode through the HIP megakernel.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c1..c5] [--extras all|none]
 
 One "step" is one decode step (one token): embedding row -> hidden state,
 barrier reset, the instruction stream, argmax over the logits, token write -
@@ -21,6 +21,12 @@ Workloads (random bf16 weights N(0, 0.02) from seed 0, RMSNorm weights 1):
 The 1B weights come from the CPU generator; the 8B weights (7.5 G parameters) and the long KV
 pre-fills are drawn by the GPU's generator, which takes seconds instead of minutes.  The prompt
 prefill runs on the GPU, outside the timed region, and its cache is what the CPU checker starts from.
+
+Without --workload the headline line is c2 (the configuration the metric is quoted on) and the other
+four workloads are measured in the same process, briefly (--extra-steps timed steps, --extra-cpu-steps
+steps checked on the CPU), into the `workloads` object of the line: tokens/s, step time, roofline
+fraction and token parity of each; an extra that fails leaves its error string there and the headline
+line is printed all the same.  --workload X measures X alone, in full.
 
 Prints one JSON line.  `roofline` prices the megakernel alone: algorithmic
 bytes per launch (weights + norm weights + K/V read, summed over the steps of
@@ -68,38 +74,9 @@ def algorithmic_bytes(cfg, pos: int) -> int:
     return 2 * (matrices + norms + kv)
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=64)
-    ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
-    ap.add_argument("--cpu-steps", type=int, default=-1,
-                    help="decode steps timed on the CPU checker (0 = skip; default 32 for the 1B workloads, 4 for 8B)")
-    ap.add_argument("--torch-steps", type=int, default=-1,
-                    help="decode steps also timed on the torch restatement of the Python VM, the closer stand-in for "
-                         "the reference's python_vm.py (0 = skip; default 3 for 1B, 1 for 8B)")
-    ap.add_argument("--sched", default="rr")
-    ap.add_argument("--workers", type=int, default=0, help="instruction queues (0 = one per compute unit)")
-    ap.add_argument("--partitions", type=int, default=0, help="attention partitions (0 = one per 256 positions, at most 24, or one per worker and KV head when the jobs are long)")
-    ap.add_argument("--loop", default="fused", choices=["fused", "reference"],
-                    help="fused: one launch per token (embedding row, barrier reset and argmax inside the "
-                         "megakernel); reference: the reference generator's sequence of small kernels around "
-                         "the launch")
-    ap.add_argument("--launch-steps", type=int, default=8,
-                    help="--loop fused: decode steps per megakernel launch (the token of one step starts the "
-                         "next inside the kernel); 1 = one launch per token, 0 = all steps of a phase in one launch")
-    ap.add_argument("--copy-calibration", action="store_true",
-                    help="after the timed region also run a plain 1 GiB device copy three times, so that a "
-                         "rocprofv3 --pmc run of this command holds a kernel of known traffic to scale "
-                         "FETCH_SIZE / WRITE_SIZE by")
-    args = ap.parse_args()
-
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs the decode path on ONE GPU; --gpus N with N > 1 is not supported "
-              "(batch-1 decode does not shard into independent units)", file=sys.stderr)
-        sys.exit(2)
-
+def run_workload(name: str, args, steps: int, warmup: int, cpu_steps: int, torch_steps: int) -> dict:
+    """One workload: build the model, schedule and generator, time `steps` decode steps after `warmup`,
+    check the first tokens against the CPU checker.  Returns the JSON object of the workload."""
     import torch
 
     from megakernels_amd.demos.latency.scheduler import LatencyScheduleBuilder, pick_num_attention_partitions
@@ -110,20 +87,19 @@ def main():
     from megakernels_amd.scheduler import assign_to_sms, tensorize_instructions
     from megakernels_amd.utils import get_sm_count, set_sm_count_override
 
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(1)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
-    work = WORKLOADS[args.workload]
+    work = WORKLOADS[name]
     big = work["arch"] == "8b"
     cfg = LlamaConfig.llama_8b() if big else LlamaConfig.llama_1b()
-    total_steps = args.warmup + args.steps
+    total_steps = warmup + steps
     prefill = work["prefill"]
     max_len = prefill + total_steps + 16
-    cpu_steps = args.cpu_steps if args.cpu_steps >= 0 else (4 if big else 32)
-    torch_steps = args.torch_steps if args.torch_steps >= 0 else (1 if big else 3)
+    if cpu_steps < 0:
+        cpu_steps = 4 if big else 32
+    if torch_steps < 0:
+        torch_steps = 1 if big else 3
     need_cpu_twin = cpu_steps > 0 or torch_steps > 0
     t_setup = time.time()
     extra = ExtraModelConfig(interleave_rope=True, max_len_override=max_len)
@@ -170,17 +146,17 @@ def main():
     setup_s = time.time() - t_setup
 
     # ---- warmup -------------------------------------------------------------
-    if args.warmup:
-        gen.generate(output_tokens, prompt_len=prefill, ntok=args.warmup, ntok_already_generated=1)
+    if warmup:
+        gen.generate(output_tokens, prompt_len=prefill, ntok=warmup, ntok_already_generated=1)
     torch.cuda.synchronize()
     mk_mod.check_status(device)
 
     # ---- timed region: exactly K steps --------------------------------------
     # kernel-only events: wrap the interpreter so each launch is bracketed on the launch stream
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
-    ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     steps_of_launch = []
-    plain = {name: getattr(interpreter, name) for name in ("interpret", "interpret_step", "interpret_steps")}
+    plain = {n: getattr(interpreter, n) for n in ("interpret", "interpret_step", "interpret_steps")}
 
     def timed(launch, count):
         def wrapper(*a, **kw):
@@ -196,18 +172,18 @@ def main():
     interpreter.interpret_steps = timed(plain["interpret_steps"], lambda globs, embed, token_in, tokens_out: tokens_out.numel())
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    gen.generate(output_tokens, prompt_len=prefill, ntok=args.steps, ntok_already_generated=1 + args.warmup)
+    gen.generate(output_tokens, prompt_len=prefill, ntok=steps, ntok_already_generated=1 + warmup)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    for name, fn in plain.items():
-        setattr(interpreter, name, fn)
+    for n, fn in plain.items():
+        setattr(interpreter, n, fn)
     mk_mod.check_status(device)
-    assert sum(steps_of_launch) == args.steps
+    assert sum(steps_of_launch) == steps
 
     launch_ms = [s.elapsed_time(e) for s, e, _ in zip(starts, ends, steps_of_launch)]
-    first_pos = prefill + args.warmup
-    step_bytes = [algorithmic_bytes(cfg, first_pos + i) for i in range(args.steps)]
-    bytes_per_step = sum(step_bytes) / args.steps
+    first_pos = prefill + warmup
+    step_bytes = [algorithmic_bytes(cfg, first_pos + i) for i in range(steps)]
+    bytes_per_step = sum(step_bytes) / steps
     # the roofline is quoted on the launches of the usual size (a shorter last launch, when the
     # step count does not divide, is left out of the mean)
     usual = max(steps_of_launch)
@@ -291,7 +267,7 @@ def main():
     # HBM bytes per launch measured with rocprofv3 --pmc for this workload (committed summary)
     traffic = None
     traffic_source = None
-    traffic_file = ROOT / "profiles" / f"mk_llama_kernel_{args.workload}_traffic.json"
+    traffic_file = ROOT / "profiles" / f"mk_llama_kernel_{name}_traffic.json"
     if traffic_file.exists():
         traffic_source = f"committed rocprofv3 --pmc summary profiles/{traffic_file.name} (not measured in this run)"
         measured = json.loads(traffic_file.read_text())
@@ -299,25 +275,25 @@ def main():
         per_step = (measured["fetch_bytes_per_launch"] + measured["write_bytes_per_launch"]) / measured.get("steps_per_launch", 1)
         traffic = int(per_step * usual)
 
-    result = {
+    return {
         "metric": f"batch-1 decode tokens/s ({'Llama-3.1-8B' if big else 'Llama-3.2-1B'} arch)",
-        "value": round(args.steps / elapsed, 2),
+        "value": round(steps / elapsed, 2),
         "unit": "tokens/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(elapsed / args.steps * 1e3, 4),
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": round(elapsed / steps * 1e3, 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
         "config": {
-            "workload": f"{args.workload}: {'Llama-3.1-8B' if big else 'Llama-3.2-1B'} architecture, random-init bf16 "
+            "workload": f"{name}: {'Llama-3.1-8B' if big else 'Llama-3.2-1B'} architecture, random-init bf16 "
                         f"weights (seed 0, {'GPU' if big else 'CPU'} generator), batch 1, "
                         + (f"32-token prompt prefilled on the GPU, " if work["kv"] == "prompt" else
                            f"KV pre-filled to {prefill} positions with seeded N(0,1), ")
-                        + f"greedy decode of {args.steps} timed tokens from position {first_pos}",
+                        + f"greedy decode of {steps} timed tokens from position {first_pos}",
             "workers": workers,
             "attention_partitions": partitions,
             "assignment": args.sched,
@@ -333,7 +309,7 @@ def main():
             "frac": round(achieved_gbps / HBM_PEAK_GBPS, 4),
             "traffic": traffic,
             "traffic_source": traffic_source,
-            "kernel": "mk_llama_kernel<8,4,128>" if big else "mk_llama_kernel<4,4,64>",
+            "kernel": "mk_llama_kernel<8,4,128,false>" if big else "mk_llama_kernel<4,4,64,false>",
             "kernel_us": round(kernel_ms_mean * 1e3, 2),
             "kernel_us_per_step": round(kernel_ms_mean * 1e3 / usual, 2),
             "launches_timed": len(usual_ms),
@@ -341,9 +317,86 @@ def main():
         },
         "cpu_baseline": cpu_baseline,
         "parity": parity,
-        "whole_step_roofline_frac": round(bytes_per_step / (elapsed / args.steps) / 1e9 / HBM_PEAK_GBPS, 4),
+        "whole_step_roofline_frac": round(bytes_per_step / (elapsed / steps) / 1e9 / HBM_PEAK_GBPS, 4),
         "setup_s": round(setup_s, 1),
     }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--workload", default=None, choices=sorted(WORKLOADS),
+                    help="the workload of the headline line (default c2, the one the metric is quoted on); given "
+                         "explicitly, only that workload runs")
+    ap.add_argument("--extras", default=None, choices=["all", "none"],
+                    help="also measure the other four workloads of the baseline, briefly, into the `workloads` object "
+                         "of the same JSON line (default: all when --workload is not given)")
+    ap.add_argument("--extra-steps", type=int, default=16, help="timed decode steps of each extra workload")
+    ap.add_argument("--extra-cpu-steps", type=int, default=2, help="decode steps of each extra workload checked on the CPU")
+    ap.add_argument("--cpu-steps", type=int, default=-1,
+                    help="decode steps timed on the CPU checker (0 = skip; default 32 for the 1B workloads, 4 for 8B)")
+    ap.add_argument("--torch-steps", type=int, default=-1,
+                    help="decode steps also timed on the torch restatement of the Python VM, the closer stand-in for "
+                         "the reference's python_vm.py (0 = skip; default 3 for 1B, 1 for 8B)")
+    ap.add_argument("--sched", default="rr")
+    ap.add_argument("--workers", type=int, default=0, help="instruction queues (0 = one per compute unit)")
+    ap.add_argument("--partitions", type=int, default=0, help="attention partitions (0 = one per 256 positions, at most 24, or one per worker and KV head when the jobs are long)")
+    ap.add_argument("--loop", default="fused", choices=["fused", "reference"],
+                    help="fused: one launch per token (embedding row, barrier reset and argmax inside the "
+                         "megakernel); reference: the reference generator's sequence of small kernels around "
+                         "the launch")
+    ap.add_argument("--launch-steps", type=int, default=8,
+                    help="--loop fused: decode steps per megakernel launch (the token of one step starts the "
+                         "next inside the kernel); 1 = one launch per token, 0 = all steps of a phase in one launch")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="after the timed region also run a plain 1 GiB device copy three times, so that a "
+                         "rocprofv3 --pmc run of this command holds a kernel of known traffic to scale "
+                         "FETCH_SIZE / WRITE_SIZE by")
+    args = ap.parse_args()
+
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs the decode path on ONE GPU; --gpus N with N > 1 is not supported "
+              "(batch-1 decode does not shard into independent units)", file=sys.stderr)
+        sys.exit(2)
+
+    import gc
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+
+    headline = args.workload or "c2"
+    extras = args.extras or ("all" if args.workload is None else "none")
+    result = run_workload(headline, args, args.steps, args.warmup, args.cpu_steps, args.torch_steps)
+    if extras == "all":
+        # the other workloads of the baseline in the same process, briefly: the figures a reader needs
+        # to place them (throughput, step time, roofline fraction, token parity), not the full record
+        result["workloads"] = {}
+        for name in sorted(WORKLOADS):
+            if name == headline:
+                continue
+            gc.collect()
+            torch.cuda.empty_cache()
+            try:
+                extra_steps = max(args.launch_steps, args.extra_steps)
+                r = run_workload(name, args, extra_steps, max(args.launch_steps, 8), args.extra_cpu_steps, 0)
+                result["workloads"][name] = {
+                    "workload": r["config"]["workload"],
+                    "value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"],
+                    "steps": r["steps"], "attention_partitions": r["config"]["attention_partitions"],
+                    "roofline": {"frac": r["roofline"]["frac"], "achieved": r["roofline"]["achieved"], "unit": "GB/s",
+                                 "kernel": r["roofline"]["kernel"], "kernel_us_per_step": r["roofline"]["kernel_us_per_step"],
+                                 "launches_timed": r["roofline"]["launches_timed"]},
+                    "cpu_baseline": {k: r["cpu_baseline"][k] for k in ("value", "unit", "cores", "kind", "sample")} if r["cpu_baseline"] else None,
+                    "parity": r["parity"],
+                    "setup_s": r["setup_s"],
+                }
+            except Exception as e:  # the headline line is printed whatever happens to an extra
+                result["workloads"][name] = {"error": f"{type(e).__name__}: {e}"}
     print(json.dumps(result))
 
 

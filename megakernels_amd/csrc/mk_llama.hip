@@ -123,12 +123,29 @@ constexpr int rows_in_flight(int wanted) { return KC <= 4 ? wanted : (wanted < M
 #define MK_PARK_UPGATE 1            // long-waiting O-proj + up/gate workers park up/gate's last rows in LDS
 #endif
 #ifndef MK_PARK_DOWN
-#define MK_PARK_DOWN 1              // ... and the last row per wave of the down projection that follows
+#define MK_PARK_DOWN 1              // ... and the last rows per wave of the down projection that follows
+#endif
+#ifndef MK_PARK_ALL
+#define MK_PARK_ALL 0               // 1: also the workers that come to O-proj + up/gate from attention park rows
 #endif
 #ifndef MK_POLL_SLEEP
 #define MK_POLL_SLEEP 10            // units of 64 clocks between two looks at a dependency
 #endif
-constexpr int kParkBytes = MK_PARK_DOWN ? kConsumerWaves * 4096 : 16;  // one more parked row per wave, outside the score buffer
+// Weight rows parked in LDS (requested long before their instruction, straight from HBM into LDS) live
+// in one region that starts with the attention score buffer and continues behind it.  With eight
+// consumer waves the registers hold six of a wave's eight up/gate rows: the other two are parked in the
+// score buffer and one row per wave of the following down projection behind it.  With more consumer
+// waves all up/gate rows fit the registers, and the region takes rows of the down projection: behind
+// the first 16 KB, where the jointly executed down projection keeps its activation vector.
+#ifndef MK_PARK_DOWN_ROWS
+#define MK_PARK_DOWN_ROWS (MK_CONSUMER_WAVES <= 8 ? 1 : 2)
+#endif
+constexpr int kParkedUpgateRows = MK_PARK_UPGATE && kConsumerWaves <= 8 ? 2 : 0;  // per wave
+constexpr int kParkedDownRows = MK_PARK_DOWN ? MK_PARK_DOWN_ROWS : 0;             // per wave
+constexpr int kScoreBytes = kScoreCap * kGqa * 4;
+constexpr int kParkDownOffset = kConsumerWaves <= 8 ? kScoreBytes : 16 * 1024;     // into the region
+constexpr int kParkRegionBytes = kParkDownOffset + kConsumerWaves * kParkedDownRows * 4096;
+constexpr int kParkBytes = kParkRegionBytes > kScoreBytes ? kParkRegionBytes - kScoreBytes : 16;  // behind the score buffer
 #define AG __HIP_MEMORY_SCOPE_AGENT
 
 // ---------------------------------------------------------------------------------------------
@@ -174,6 +191,7 @@ struct Consts {
     int cols;                       // columns of `barriers`: query + key + value heads
     int pad_cols;                   // padded per-head counters per (layer, row)
     int down_jobs, o_jobs;          // arrivals that complete barrier rows 5 and 3
+    int shard_stride, replica_stride;  // ints from one shard / one replica of a sharded counter to the next
 };
 // A matvec instruction (opcodes 1, 4, 5, 6) decoded once per launch: where its weight rows live.
 // ntasks < 0: the instruction is malformed.
@@ -185,6 +203,17 @@ struct alignas(16) SlotDesc {
     int ntasks, first_row;
 };
 static_assert(sizeof(SlotDesc) == 32, "two 16-byte LDS reads");
+// Where an instruction's dependency counter and the counter it signals live (opcodes 1, 4, 5, 6, 7),
+// worked out once per launch: the first look at a dependency and the signal after the store
+// acknowledgement then need one LDS round trip, not a chain of them.
+struct alignas(16) SyncDesc {
+    uint64_t poll_base;             // lane l < kShards looks at (int *)poll_base + l * shard_stride; 0: nothing to wait for
+    uint64_t bar_word;              // lane kShards looks at the counter's word in `barriers`
+    uint64_t signal_base;           // this worker's shard of the counter the instruction signals, first replica
+    int target;                     // arrivals that satisfy the dependency
+    int pad;
+};
+static_assert(sizeof(SyncDesc) == 32, "two 16-byte LDS reads");
 
 struct Smem {
     int abort;                      // set once, never cleared during a launch
@@ -194,15 +223,24 @@ struct Smem {
     Consts k;
     mk_llama_args args;             // the launch arguments, read from here by every instruction
     int flags[16];                  // scratch of the end-of-step reduction
-    alignas(16) uint32_t x[kMaxK / 2];          // activation vector as bf16 pairs, lane layout [chunk][lane][4 dwords]
-    alignas(16) float out[kOutRows];            // matvec row results awaiting the epilogue
-    alignas(16) float wave_max[kAttnWaves][kGqa];
-    alignas(16) float wave_l[kAttnWaves][kGqa];
-    alignas(16) float wave_o[kAttnWaves][kGqa][kMaxHeadDim];
+    // the matvec instructions' hand-over buffers and attention's share their space: an instruction
+    // uses one set or the other, and nothing in them outlives an instruction
+    union {
+        struct {
+            alignas(16) uint32_t x[kMaxK / 2];          // activation vector as bf16 pairs, lane layout [chunk][lane][4 dwords]
+            alignas(16) float out[kOutRows];            // matvec row results awaiting the epilogue
+        };
+        struct {
+            alignas(16) float wave_max[kAttnWaves][kGqa];
+            alignas(16) float wave_l[kAttnWaves][kGqa];
+            alignas(16) float wave_o[kAttnWaves][kGqa][kMaxHeadDim];
+        };
+    };
     alignas(16) float scores[kScoreCap][kGqa];  // attention: one partition's scores, then probabilities
-    alignas(16) unsigned char park[kParkBytes];  // a weight row per wave parked for a later instruction
-    int parked_slot;                               // the instruction whose last row per wave lies in `park`, or -1
+    alignas(16) unsigned char park[kParkBytes];  // the parked rows' region continues here
+    int parked_slot;                               // the down projection whose last rows per wave are parked, or -1
     alignas(16) SlotDesc desc[kQueueSlots];        // the matvec instructions of the window, decoded
+    alignas(16) SyncDesc sync[kQueueSlots];        // ... and where their counters live
     alignas(16) int queue[kQueueSlots][MK_INSTRUCTION_WORDS];  // a window of this worker's instructions
 };
 static_assert(offsetof(Smem, x) % 16 == 0 && offsetof(Smem, wave_max) % 16 == 0 && offsetof(Smem, wave_l) % 16 == 0 &&
@@ -210,6 +248,7 @@ static_assert(offsetof(Smem, x) % 16 == 0 && offsetof(Smem, wave_max) % 16 == 0 
               "128-bit LDS accesses need 16-byte aligned members");
 
 static_assert(sizeof(Smem) <= 160 * 1024, "LDS budget");
+static_assert(offsetof(Smem, park) == offsetof(Smem, scores) + sizeof(Smem::scores), "the parked rows' region is contiguous");
 static_assert(sizeof(Smem) > 80 * 1024, "must keep a second workgroup off the CU");
 
 // ---------------------------------------------------------------------------------------------
@@ -600,6 +639,39 @@ __device__ bool poll_counters(const Ctx &c, const int *ptr, const int *in_barrie
     return poll_wait(c, poll_issue(c, ptr, in_barriers), sum_mode, target, []() {});
 }
 
+// The decoded counters of the instruction in the context's slot, as scalars.
+struct SyncInfo {
+    const int *poll_base, *bar_word;
+    int *signal_base;
+    int target;
+};
+__device__ __forceinline__ SyncInfo sync_info(const Ctx &c) {
+    const MK_LDS u32x4 *src = (const MK_LDS u32x4 *)&c.sm->sync[c.slot];
+    const u32x4 lo = src[0], hi = src[1];
+    auto ptr = [](uint32_t l, uint32_t h) {
+        return (int *)(uintptr_t)(((uint64_t)(uint32_t)uni((int)h) << 32) | (uint32_t)uni((int)l));
+    };
+    return SyncInfo{ptr(lo.x, lo.y), ptr(lo.z, lo.w), ptr(hi.x, hi.y), uni((int)hi.z)};
+}
+// first look at a sharded dependency counter: lanes 0 .. kShards - 1 one shard each, lane kShards the
+// word in `barriers` (what the counter held before the launch), lane 63 the status word
+__device__ __forceinline__ PollTicket poll_issue(const Ctx &c, const SyncInfo &sy) {
+    const int *ptr = nullptr;
+    if (sy.poll_base) {
+        if (c.lane < kShards) ptr = sy.poll_base + c.lane * uni(c.sm->k.shard_stride);
+        else if (c.lane == kShards) ptr = sy.bar_word;
+    }
+    return poll_issue(c, ptr);
+}
+// one arrival on the counter the instruction signals; the caller has waited for its stores
+__device__ __forceinline__ void signal_sharded(const Ctx &c, const SyncInfo &sy, int count) {
+    if (c.lane == 0) {
+        const int stride = uni(c.sm->k.replica_stride);
+#pragma unroll
+        for (int r = 0; r < kReplicas; r++) add_i32(sy.signal_base + (size_t)r * stride, count);
+    }
+}
+
 __device__ __forceinline__ const int *sharded_lane_ptr(const Ctx &c, int layer, int row) {
     // 256 workers reading the same 16 lines every quarter microsecond queue up at those lines'
     // memory channels; with four copies each line has a quarter of the readers
@@ -662,20 +734,25 @@ __device__ __forceinline__ float fold8(const float (&a)[8]) {
 // Sum of squares in column order: column c = lane * 8 + e accumulates its elements j * 512 + c in
 // order of j, the 512 columns are added as a balanced pairwise tree.
 template <int KC>
-__device__ __forceinline__ void rms_norm_x(uint4 (&xq)[KC], const XVec<KC> &x, const uint4 (&wraw)[KC], float eps) {
+__device__ __forceinline__ void rms_norm_x(uint4 (&xq)[KC], const uint4 (&xraw)[KC], const uint4 (&wraw)[KC], float eps) {
+    // the vector stays packed (bf16 pairs, half the registers) and is widened chunk by chunk, twice
     float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-    for (int j = 0; j < KC; j++)
+    for (int j = 0; j < KC; j++) {
+        float xv[8];
+        unpack8(xraw[j], xv);
 #pragma unroll
-        for (int e = 0; e < 8; e++) acc[e] = fmaf(x.v[j][e], x.v[j][e], acc[e]);
+        for (int e = 0; e < 8; e++) acc[e] = fmaf(xv[e], xv[e], acc[e]);
+    }
     const float mean = wave_tree_sum_uniform(fold8(acc)) / (float)(KC * 512);
     const float inv = 1.0f / sqrtf(mean + eps);
 #pragma unroll
     for (int j = 0; j < KC; j++) {
-        float wv[8], y[8];
+        float wv[8], xv[8], y[8];
         unpack8(wraw[j], wv);
+        unpack8(xraw[j], xv);
 #pragma unroll
-        for (int e = 0; e < 8; e++) y[e] = wv[e] * mkm::round_bf16(x.v[j][e] * inv);
+        for (int e = 0; e < 8; e++) y[e] = wv[e] * mkm::round_bf16(xv[e] * inv);
         xq[j].x = mkm::pack_bf16(y[0], y[1]);
         xq[j].y = mkm::pack_bf16(y[2], y[3]);
         xq[j].z = mkm::pack_bf16(y[4], y[5]);
@@ -912,7 +989,7 @@ struct MatvecDesc {
 // (t % 16) / G of the job's rows, column group t % G; a wave's tasks (t = wave mod 8) all have column
 // group wave % G, so the wave keeps that group's slice of the activation vector in registers.
 __host__ __device__ constexpr bool joint_groups(uint32_t flags, int G, int in_dim) {
-    return (flags & MK_FLAG_JOINT_RESIDUAL) != 0 && G > 1 && 16 % G == 0 && kConsumerWaves % G == 0 &&
+    return (flags & MK_FLAG_JOINT_RESIDUAL) != 0 && G > 1 && 16 % G == 0 && G <= 4 &&
            (size_t)in_dim * 2 <= sizeof(Smem::scores);
 }
 
@@ -981,6 +1058,53 @@ __device__ __forceinline__ void decode_matvec(SmemPtr sm, int slot, ArgsRef a) {
     dst[1] = u32x4{d.w0_bytes, d.row_bytes, (uint32_t)d.ntasks, (uint32_t)d.first_row};
 }
 
+// Where the counters of the instruction in queue slot `slot` live (opcodes 1, 4, 5, 6, 7; executed once
+// per launch by one thread per slot).  An instruction whose layer is out of range gets no counters; its
+// handler refuses it before it looks at them.
+__device__ __forceinline__ void decode_sync(SmemPtr sm, int slot, ArgsRef a) {
+    const InsPtr ins = sm->queue[slot];
+    const int opcode = ins[0], L = a.num_layers;
+    const int layer = opcode == 7 ? L - 1 : ins[1];
+    int wait_layer = -1, wait_row = 2, target = 0, signal_layer = -1, signal_row = 2;
+    if (layer >= 0 && layer < L) {
+        const int down_jobs = (a.intermediate_size / a.matvec_reduction_size) * (a.hidden_size / 16);
+        switch (opcode) {
+        case 1:  // the previous layer's down projection (python_vm.py:176)
+            if (layer > 0) { wait_layer = layer - 1; wait_row = 5; target = down_jobs; }
+            break;
+        case 4:  // all heads' attention output (python_vm.py:88-95); signals row 3
+            wait_layer = layer; wait_row = 2; target = a.num_attention_heads;
+            signal_layer = layer; signal_row = 3;
+            break;
+        case 5:  // the O projection (python_vm.py:132); signals row 4
+            wait_layer = layer; wait_row = 3; target = (a.hidden_size / a.matvec_reduction_size) * (a.hidden_size / 16);
+            signal_layer = layer; signal_row = 4;
+            break;
+        case 6:  // up / gate (python_vm.py:110); signals row 5
+            wait_layer = layer; wait_row = 4; target = a.intermediate_size / 16;
+            signal_layer = layer; signal_row = 5;
+            break;
+        default:  // 7: the last layer's down projection (python_vm.py:255)
+            wait_layer = layer; wait_row = 5; target = down_jobs;
+            break;
+        }
+    }
+    const WsLayout w = ws_layout(L, a.hidden_size, a.intermediate_size, a.matvec_reduction_size);
+    int *const shards = static_cast<int *>(a.workspace) + w.shards;
+    const int cols = a.num_attention_heads + 2 * a.num_kv_heads;
+    const int replica = ((int)blockIdx.x / kShards) % kReplicas, shard = (int)blockIdx.x & (kShards - 1);
+    uint64_t poll_base = 0, bar_word = 0, signal_base = 0;
+    if (wait_layer >= 0) {
+        poll_base = (uint64_t)(uintptr_t)(shards + ((size_t)replica * kShards * L + wait_layer) * kHotRows + (wait_row - 2));
+        bar_word = (uint64_t)(uintptr_t)(a.barriers + ((size_t)wait_layer * MK_BARRIER_ROWS + wait_row) * cols);
+    }
+    if (signal_layer >= 0)
+        signal_base = (uint64_t)(uintptr_t)(shards + ((size_t)shard * L + signal_layer) * kHotRows + (signal_row - 2));
+    MK_LDS u32x4 *dst = (MK_LDS u32x4 *)&sm->sync[slot];
+    dst[0] = u32x4{(uint32_t)poll_base, (uint32_t)(poll_base >> 32), (uint32_t)bar_word, (uint32_t)(bar_word >> 32)};
+    dst[1] = u32x4{(uint32_t)signal_base, (uint32_t)(signal_base >> 32), (uint32_t)target, 0u};
+}
+
 // The decoded form of the matvec instruction in `slot`; false: the instruction is malformed.
 __device__ __forceinline__ bool describe_matvec(SmemPtr sm, int slot, int opcode, MatvecDesc &d) {
     const MK_LDS u32x4 *src = (const MK_LDS u32x4 *)&sm->desc[slot];
@@ -1026,21 +1150,21 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
     const int layer = ins[1], start = ins[2], end = ins[3];
     const int hid = a.hidden_size, D = a.head_dim, H = a.num_attention_heads, KVH = a.num_kv_heads;
     const int nblk = end > start ? end - start : 0;
-    const int down_jobs = c.sm->k.down_jobs;
     const int k_start = H * D, v_start = k_start + KVH * D;
     constexpr int kPre = 2;
     float rot[kPre][4] = {{1.0f, 1.0f, 0.0f, 0.0f}, {1.0f, 1.0f, 0.0f, 0.0f}};
     const bool prefetched = nblk * 8 <= kPre * 64;
     PollTicket ticket = {nullptr, 0, 0};
+    const SyncInfo sy = sync_info(c);
     uint4 wraw[KC];
     return controller_sequence(
         c,
         [&]() {
-            if (layer > 0) ticket = poll_issue(c, sharded_lane_ptr(c, layer - 1, 5));
+            ticket = poll_issue(c, sy);
             if (nblk > 0) load_row<KC>(wraw, a.attn_norm_weights + (size_t)layer * hid, c.lane);
         },
         [&](auto release) {
-            if (layer > 0 && !poll_wait(c, ticket, true, down_jobs, release)) return false;
+            if (layer > 0 && !poll_wait(c, ticket, true, sy.target, release)) return false;
             trace_event(c, kEvDepReady, MK_TIMING_DONE_GMEM_WAIT);
             if (nblk > 0) {
                 // layer 0 of a launch that was given a token reads the embedding row itself; the
@@ -1048,15 +1172,18 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
                 // reader of hidden_states waits, through attention, for this worker's signal)
                 const bool from_table = layer == 0 && a.token_in != nullptr;
                 const uint16_t *src = from_table ? a.embed_table + (size_t)c.sm->token * hid : a.hidden_states;
-                XVec<KC> x;
-                load_x<KC>(x, src, c.lane);
+                uint4 x[KC];
+                load_xq<KC>(x, src, c.lane);
                 release();
                 if (from_table && start == 0) {
 #pragma unroll
-                    for (int j = 0; j < KC; j++)
-#pragma unroll
-                        for (int e = 0; e < 8; e += 2)
-                            st_u32(a.hidden_states + j * 512 + c.lane * 8 + e, mkm::pack_bf16(x.v[j][e], x.v[j][e + 1]));
+                    for (int j = 0; j < KC; j++) {
+                        uint16_t *dst = a.hidden_states + j * 512 + c.lane * 8;
+                        st_u32(dst, x[j].x);
+                        st_u32(dst + 2, x[j].y);
+                        st_u32(dst + 4, x[j].z);
+                        st_u32(dst + 6, x[j].w);
+                    }
                 }
                 uint4 xq[KC];
                 rms_norm_x<KC>(xq, x, wraw, a.rms_norm_eps);
@@ -1158,8 +1285,7 @@ __device__ __forceinline__ bool control_matvec_add(const Ctx &c) {
     // column groups executed jointly by this job (0: its own group only), as decoded
     const int joint = uni((int)((const MK_LDS uint32_t *)&c.sm->desc[c.slot])[2]);
     const uint16_t *vec = (is_down ? a.silu_out : a.attn_out) + (joint ? 0 : (size_t)group * R);
-    const int wait_row = is_down ? 4 : 2;
-    const int wait_target = is_down ? a.intermediate_size / 16 : a.num_attention_heads;
+    const SyncInfo sy = sync_info(c);
     uint16_t *resid = a.hidden_states;
     // One lane per pair of adjacent residual rows.  Alone, a job owns all 16 rows of its blocks; in
     // joint execution it owns 16 / G rows of each, starting at row group * 16 / G.
@@ -1183,14 +1309,14 @@ __device__ __forceinline__ bool control_matvec_add(const Ctx &c) {
     PollTicket ticket = {nullptr, 0, 0};
     return controller_sequence(
         c,
-        [&]() { ticket = poll_issue(c, sharded_lane_ptr(c, layer, wait_row)); },
+        [&]() { ticket = poll_issue(c, sy); },
         [&](auto release) {
-            if (!poll_wait(c, ticket, true, wait_target, release)) return false;
+            if (!poll_wait(c, ticket, true, sy.target, release)) return false;
             trace_event(c, kEvDepReady, MK_TIMING_DONE_GMEM_WAIT);
             if (nblk > 0) {
                 if (joint) {
                     // all column groups' slices of the vector, into the attention score buffer (idle here)
-                    constexpr int kMaxJoint = kConsumerWaves < 4 ? kConsumerWaves : 4;
+                    constexpr int kMaxJoint = 4;
                     uint4 xq[kMaxJoint][KC];
 #pragma unroll
                     for (int g = 0; g < kMaxJoint; g++)
@@ -1294,7 +1420,7 @@ __device__ __forceinline__ bool control_matvec_add(const Ctx &c) {
             trace_store_issue(c);
             if (guards_data) wait_stores();
             trace_store_done(c);
-            signal_sharded(c, layer, is_down ? 5 : 3, nblk);
+            signal_sharded(c, sy, nblk);
             trace_signalled(c);
         });
 }
@@ -1309,21 +1435,21 @@ __device__ __forceinline__ bool control_upgate(const Ctx &c) {
     ArgsRef a = c.sm->args;
     const int layer = ins[1], n = ins[2];
     const int hid = a.hidden_size;
-    const int o_jobs = c.sm->k.o_jobs;
+    const SyncInfo sy = sync_info(c);
     PollTicket ticket = {nullptr, 0, 0};
     uint4 wraw[KC];
     return controller_sequence(
         c,
         [&]() {
-            ticket = poll_issue(c, sharded_lane_ptr(c, layer, 3));
+            ticket = poll_issue(c, sy);
             if (n > 0) load_row<KC>(wraw, a.mlp_norm_weights + (size_t)layer * hid, c.lane);
         },
         [&](auto release) {
-            if (!poll_wait(c, ticket, true, o_jobs, release)) return false;
+            if (!poll_wait(c, ticket, true, sy.target, release)) return false;
             trace_event(c, kEvDepReady, MK_TIMING_DONE_GMEM_WAIT);
             if (n > 0) {
-                XVec<KC> x;
-                load_x<KC>(x, a.hidden_states, c.lane);
+                uint4 x[KC];
+                load_xq<KC>(x, a.hidden_states, c.lane);
                 release();
                 uint4 xq[KC];
                 rms_norm_x<KC>(xq, x, wraw, a.rms_norm_eps);
@@ -1344,7 +1470,7 @@ __device__ __forceinline__ bool control_upgate(const Ctx &c) {
             trace_store_issue(c);
             wait_stores();
             trace_store_done(c);
-            signal_sharded(c, layer, 4, n);
+            signal_sharded(c, sy, n);
             trace_signalled(c);
         });
 }
@@ -1405,10 +1531,13 @@ __device__ __forceinline__ void park_rows(const Ctx &c, MK_LDS unsigned char *sl
 // earlier request and are taken from there; the rows before them stream as usual.
 // where this wave's activation vector lies in LDS: the common buffer, or - for a jointly executed
 // column-group job - the slice of the wave's column group in the attention score buffer
+// (task t of such a job works on column group t mod G: the same for all tasks of a wave when the
+// number of consumer waves is a multiple of G, else the wave fetches the slice per task)
+constexpr bool kJointSlicePerTask = kConsumerWaves % 4 != 0;
 template <int KC>
-__device__ __forceinline__ const MK_LDS uint32_t *x_source(const Ctx &c, const MatvecDesc &d) {
+__device__ __forceinline__ const MK_LDS uint32_t *x_source(const Ctx &c, const MatvecDesc &d, int task) {
     if ((d.opcode == 4 || d.opcode == 6) && d.gate_delta > 0)
-        return (const MK_LDS uint32_t *)&c.sm->scores[0][0] + (c.wave & ((int)d.gate_delta - 1)) * (KC * 256);
+        return (const MK_LDS uint32_t *)&c.sm->scores[0][0] + (task & ((int)d.gate_delta - 1)) * (KC * 256);
     return (const MK_LDS uint32_t *)c.sm->x;
 }
 
@@ -1418,11 +1547,14 @@ __device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&pool)[NBUF][K
     constexpr int PF = Map::size;
     if (!barrier_inputs_ready(c, true)) return false;
     XPairs<KC> x;
-    if (d.ntasks > 0) x_from_lds<KC>(x, x_source<KC>(c, d), c.lane);
+    const bool per_task = kJointSlicePerTask && (d.opcode == 4 || d.opcode == 6) && d.gate_delta > 0;
+    if (d.ntasks > 0 && !per_task) x_from_lds<KC>(x, x_source<KC>(c, d, c.wave), c.lane);
     trace_consumer_first_use(c);
     auto consume = [&](const uint4 (&src)[KC], int i) {
+        const int task = c.wave + i * kConsumerWaves;
+        if (per_task) x_from_lds<KC>(x, x_source<KC>(c, d, task), c.lane);
         const float y = mkm::round_bf16(dot_row<KC>(src, x));
-        if (c.lane == 0) c.sm->out[c.wave + i * kConsumerWaves] = y;
+        if (c.lane == 0) c.sm->out[task] = y;
     };
     const int parked_first = mine > PARKED ? mine - PARKED : 0;  // rows from here on are in LDS
     const int streamed = PARKED > 0 ? parked_first : mine;
@@ -1509,7 +1641,8 @@ __device__ __forceinline__ bool matvec_impl(SmemPtr lds, int slot, int *refusal)
     wg_barrier();  // entry: the controller's first requests are out
     trace_first_load(c);
     request_rows<KC, Map>(c, pool, d, 0, mine > PARKED ? mine - PARKED : 0);
-    const bool ok = consumer_run<KC, Map, PF, PARKED>(c, pool, d, mine, (MK_LDS const unsigned char *)lds->park + c.wave * (KC * 1024));
+    const bool ok = consumer_run<KC, Map, PF, PARKED>(
+        c, pool, d, mine, (MK_LDS const unsigned char *)&lds->scores[0][0] + kParkDownOffset + c.wave * (PARKED * KC * 1024));
     return ok;
 }
 template <bool TR, int OP, int KC, int PARKED = 0>
@@ -1530,7 +1663,7 @@ static __device__ __noinline__ int op_oproj_upgate(SmemPtr lds, int slot, int *r
     // PARK: this worker has a long wait ahead (it came here without attention work) and its up/gate
     // instruction has at most two rows per wave beyond the six buffers: those go to LDS on entry - the
     // attention score buffer is free - and up/gate then needs nothing from HBM once its dependency resolves
-    constexpr int kParked = PARK && (size_t)kConsumerWaves * 2 * KC * 1024 <= sizeof(Smem::scores) ? 2 : 0;
+    constexpr int kParked = PARK && (size_t)kConsumerWaves * kParkedUpgateRows * KC * 1024 <= sizeof(Smem::scores) ? kParkedUpgateRows : 0;
     typedef BufMap<0, 1> MapO;
     typedef BufMap<2, 3, 4, 5> MapU0;        // requested on entry
     typedef BufMap<0, 1> MapU1;              // requested when O-proj is done
@@ -1556,15 +1689,19 @@ static __device__ __noinline__ int op_oproj_upgate(SmemPtr lds, int slot, int *r
     request_rows<KC, MapU0>(co, pool, dsu, 0, stream_u, pair);
     MK_LDS unsigned char *slice = (MK_LDS unsigned char *)&lds->scores[0][0] + co.wave * (kParked * KC * 1024);
     if constexpr (PARK) {
-        park_rows<KC, kParked>(co, slice, dsu, mine_u > kParked ? mine_u - kParked : 0, mine_u, pair);
-        // and the last row per wave of a down projection that follows directly
-        MatvecDesc dsd;
-        const bool down_next = MK_PARK_DOWN && KC * 1024 * kConsumerWaves <= kParkBytes && slot + 2 < uni(lds->window_count) &&
-                               uni(lds->queue[slot + 2][0]) == 6 && describe_matvec(lds, slot + 2, 6, dsd);
-        if (!down_next) dsd = dso;
-        const int mine_d = down_next ? rows_of_wave(dsd.ntasks, co.wave) : 0;
-        park_rows<KC, 1>(co, (MK_LDS unsigned char *)lds->park + co.wave * (KC * 1024), dsd, mine_d > 0 ? mine_d - 1 : 0, mine_d, down_next);
-        if (co.lane == 0 && co.wave == 0) lds->parked_slot = down_next ? slot + 2 : -1;
+        if constexpr (kParked > 0) park_rows<KC, kParked>(co, slice, dsu, mine_u > kParked ? mine_u - kParked : 0, mine_u, pair);
+        // and the last rows per wave of a down projection that follows directly
+        if constexpr (kParkedDownRows > 0 && KC * 1024 == 4096) {
+            MatvecDesc dsd;
+            const bool down_next = slot + 2 < uni(lds->window_count) && uni(lds->queue[slot + 2][0]) == 6 &&
+                                   describe_matvec(lds, slot + 2, 6, dsd);
+            if (!down_next) dsd = dso;
+            const int mine_d = down_next ? rows_of_wave(dsd.ntasks, co.wave) : 0;
+            park_rows<KC, kParkedDownRows>(
+                co, (MK_LDS unsigned char *)&lds->scores[0][0] + kParkDownOffset + co.wave * (kParkedDownRows * KC * 1024), dsd,
+                mine_d > kParkedDownRows ? mine_d - kParkedDownRows : 0, mine_d, down_next);
+            if (co.lane == 0 && co.wave == 0) lds->parked_slot = down_next ? slot + 2 : -1;
+        }
     }
     if (!consumer_run<KC, MapO>(co, pool, dso, mine_o)) return 0;
     request_rows<KC, MapU1>(co, pool, dsu, MapU0::size, stream_u, pair);
@@ -1599,7 +1736,7 @@ static __device__ __noinline__ bool op_lm_head(SmemPtr lds, int slot, int *refus
     const int start = ins[1], end = ins[2];
     const int hid = a.hidden_size;
     if (start < 0 || end > a.vocab_size / 16) return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
-    const int down_jobs = c.sm->k.down_jobs;
+    const SyncInfo sy = c.controller ? sync_info(c) : SyncInfo{nullptr, nullptr, nullptr, 0};
     const int blocks_per_batch = kOutRows / 16;
     const WeightBuffer W = weight_buffer(a.lm_head_weights, (size_t)a.vocab_size * hid * 2);
     float best_v = -INFINITY;
@@ -1615,15 +1752,15 @@ static __device__ __noinline__ bool op_lm_head(SmemPtr lds, int slot, int *refus
             c, nblk * 16, true, [&](int t) { return RowRef{W, (uint32_t)(b0 * 16 + t) * (uint32_t)hid * 2u}; },
             [&]() {
                 if (!first) return;
-                ticket = poll_issue(c, sharded_lane_ptr(c, a.num_layers - 1, 5));
+                ticket = poll_issue(c, sy);
                 load_row<KC>(wraw, a.lm_head_norm_weights, c.lane);
             },
             [&](auto release) {
                 if (!first) return true;  // the activation vector stays in LDS between batches
-                if (!poll_wait(c, ticket, true, down_jobs, release)) return false;
+                if (!poll_wait(c, ticket, true, sy.target, release)) return false;
                 trace_event(c, kEvDepReady, MK_TIMING_DONE_GMEM_WAIT);
-                XVec<KC> x;
-                load_x<KC>(x, a.hidden_states, c.lane);
+                uint4 x[KC];
+                load_xq<KC>(x, a.hidden_states, c.lane);
                 release();
                 uint4 xq[KC];
                 rms_norm_x<KC>(xq, x, wraw, a.rms_norm_eps);
@@ -2229,6 +2366,7 @@ static __device__ __noinline__ void fetch_window(SmemPtr sm, int base) {
     for (int slot = tid; slot < count; slot += kThreads) {
         const int opcode = sm->queue[slot][0];
         if (opcode == 1 || (opcode >= 4 && opcode <= 6)) decode_matvec(sm, slot, a);
+        if (opcode == 1 || (opcode >= 4 && opcode <= 7)) decode_sync(sm, slot, a);
     }
     wg_barrier();
 }
@@ -2435,6 +2573,8 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
         sm->k.pad_cols = pad_cols(a.hidden_size);
         sm->k.down_jobs = (a.intermediate_size / a.matvec_reduction_size) * (a.hidden_size / 16);
         sm->k.o_jobs = (a.hidden_size / a.matvec_reduction_size) * (a.hidden_size / 16);
+        sm->k.shard_stride = a.num_layers * kHotRows;
+        sm->k.replica_stride = kShards * a.num_layers * kHotRows;
     }
     // A launch covers one decode step, or `num_steps` of them back to back: the token a step
     // produces starts the next one, at the next position.
@@ -2491,8 +2631,9 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
                             // the wait is too short for it to pay) and the up/gate instruction is small
                             // enough (two list entries: eight rows per wave)
                             const int entries = uni(sm->queue[slot + 1][2]);
-                            const bool park = MK_PARK_UPGATE && !uni(sm->args.skip_attn_reduction) &&
-                                              (slot == 0 || uni(sm->queue[slot - 1][0]) != 2) && entries >= 0 && entries <= 2;
+                            const bool park = (kParkedUpgateRows > 0 || kParkedDownRows > 0) && !uni(sm->args.skip_attn_reduction) &&
+                                              (MK_PARK_ALL || slot == 0 || uni(sm->queue[slot - 1][0]) != 2) && entries >= 0 &&
+                                              (kParkedUpgateRows == 0 || entries <= 2);
                             const int executed = uni(park ? op_oproj_upgate<TR, KC_HID, true>(sm, slot, &refusal)
                                                           : op_oproj_upgate<TR, KC_HID, false>(sm, slot, &refusal));
                             ok = executed > 0;
@@ -2504,9 +2645,9 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
                     break;
                 case 5: ok = uni((int)op_matvec<TR, 5, KC_HID>(sm, slot, &refusal)) != 0; break;
                 case 6:
-                    if constexpr (KC_HID == KC_RED && MK_PAIR_OPROJ_UPGATE && MK_PARK_UPGATE && MK_PARK_DOWN) {
+                    if constexpr (KC_HID == KC_RED && MK_PAIR_OPROJ_UPGATE && kParkedDownRows > 0) {
                         if (uni(sm->parked_slot) == slot) {
-                            ok = uni((int)op_matvec<TR, 6, KC_RED, 1>(sm, slot, &refusal)) != 0;
+                            ok = uni((int)op_matvec<TR, 6, KC_RED, kParkedDownRows>(sm, slot, &refusal)) != 0;
                             break;
                         }
                     }
