@@ -106,7 +106,10 @@ enum {
 typedef struct mk_llama_args {
     /* VM state */
     int32_t *barriers;              /* [L, 10, H + 2 KVH]; read-modify-write */
-    const int32_t *instructions;    /* [num_workers, num_slots, 32] */
+    const int32_t *instructions;    /* [num_workers, num_slots, 32]; a worker runs its row in order, so no
+                                       instruction may sit behind one that (transitively) waits for it - which,
+                                       without MK_FLAG_JOINT_RESIDUAL, includes: the job of a residual projection's
+                                       last column group waits for the other groups' jobs of its row blocks */
     int32_t *timings;               /* [num_workers, num_slots, 128]; may be NULL */
     /* weights */
     const uint16_t *qkv_weights;          /* [L, (H + 2 KVH) D, hidden] */
@@ -155,9 +158,10 @@ typedef struct mk_llama_args {
     int64_t *token_out;                   /* device; receives argmax(logits), first index on ties */
     /* Optional: several decode steps in one launch (no counterpart in the reference, which launches
      * once per token).  num_steps > 1 needs embed_table, token_in, token_out and
-     * MK_FLAG_RESET_BARRIERS; step s runs at position pos_id + s, starts from the token of step s - 1
-     * (*token_in for s = 0) and writes its token to token_out[s], so token_out holds num_steps
-     * entries.  0 and 1 both mean one step. */
+     * MK_FLAG_RESET_BARRIERS, and k_cache / v_cache aligned to 128 bytes (rows written by one step are read
+     * by the next with cached loads, so no cache line may hold bytes of two rows); step s runs at position
+     * pos_id + s, starts from the token of step s - 1 (*token_in for s = 0) and writes its token to
+     * token_out[s], so token_out holds num_steps entries.  0 and 1 both mean one step. */
     int32_t num_steps;
     int32_t reserved0;                    /* keep zero */
 } mk_llama_args;

@@ -2794,6 +2794,11 @@ int validate(const mk_llama_args &a, KernelFn *kernel) {
     if (a.num_steps > 1) {
         if (!a.token_in || !a.token_out || !(a.flags & MK_FLAG_RESET_BARRIERS))
             return fail(-3, "several steps per launch need token_in, token_out and MK_FLAG_RESET_BARRIERS");
+        // K / V rows that an earlier step of the launch wrote are read with ordinary cached loads, which is
+        // sound as long as no cache line holds bytes of two (position, head) rows: a row's line must not
+        // have been fetched, as a neighbour's, before the step that writes it
+        if ((uintptr_t)a.k_cache % 128 || (uintptr_t)a.v_cache % 128)
+            return fail(-2, "several steps per launch need k_cache and v_cache aligned to 128 bytes");
         const long long last = (long long)a.pos_id + a.num_steps - 1;
         if (last >= a.kv_max_len || last >= a.rope_positions)
             return fail(-4, "%d steps from position %d run past the KV cache (%d) or rope table (%d)", a.num_steps,

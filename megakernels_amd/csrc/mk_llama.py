@@ -19,7 +19,9 @@ import torch
 import os
 
 _HERE = Path(__file__).resolve().parent
-# MK_LLAMA_LIB selects another build of the same ABI (used when comparing kernel variants)
+# MK_LLAMA_LIB selects another build of the same ABI (for comparing kernel variants).  A library that
+# is not the one built next to this file is announced on stderr when it is loaded, so that it cannot
+# stand in for the product unnoticed.
 LIBRARY = Path(os.environ.get("MK_LLAMA_LIB", _HERE / "libmk_llama.so"))
 
 _P = ctypes.c_void_p
@@ -61,6 +63,7 @@ record_timings = False
 # per-GPU array and this module allocates nothing for a launch
 static_scratch = False
 _static_scratch_ptrs: dict[int, int] = {}
+_static_status_pending: dict[int, bool] = {}   # a static launch whose failure, if any, has not been reported yet
 # MK_FLAG_JOINT_RESIDUAL for launches that do not say (`joint_residual=` of mk_llama): None = set it
 # when the instruction tensor qualifies, False = never (every column-group job runs on its own)
 joint_residual_default = None
@@ -73,6 +76,10 @@ def load_library():
             raise RuntimeError(
                 f"{LIBRARY} is missing: build it with `python {_HERE / 'build.py'}` (needs hipcc)"
             )
+        if LIBRARY.resolve() != (_HERE / "libmk_llama.so").resolve():
+            import sys
+
+            print(f"mk_llama: MK_LLAMA_LIB is set - loading {LIBRARY} instead of {_HERE / 'libmk_llama.so'}", file=sys.stderr)
         lib = ctypes.CDLL(str(LIBRARY))
         lib.mk_llama_launch.argtypes = [ctypes.POINTER(MkLlamaArgs), _P]
         lib.mk_llama_launch.restype = ctypes.c_int
@@ -269,8 +276,11 @@ def mk_llama(
         with torch.cuda.device(barriers.device):
             where = _P()
             rc = lib.mk_llama_launch_static(ctypes.byref(a), ctypes.c_void_p(stream.cuda_stream), ctypes.byref(where))
-        if rc == 0:
+        if where.value:
+            # (every static launch clears the part of the array it uses, status included, so what is
+            # read from it afterwards belongs to this launch)
             _static_scratch_ptrs[barriers.device.index] = where.value
+            _static_status_pending[barriers.device.index] = True
     else:
         rc = lib.mk_llama_launch(ctypes.byref(a), ctypes.c_void_p(stream.cuda_stream))
     if rc != 0:
@@ -304,13 +314,14 @@ def read_status(device=None, stream=None):
     # the library's own array (launches with static_scratch): every such launch clears what it uses
     # first, so a recorded failure needs no clean-up here
     where = _static_scratch_ptrs.get(device.index)
-    if where and result[0] == 0:
+    if where and _static_status_pending.get(device.index):
         rc = lib.mk_llama_read_status(ctypes.c_void_p(where), ctypes.c_void_p(stream.cuda_stream), ctypes.byref(out))
         if rc != 0:
             raise RuntimeError(f"mk_llama_read_status failed: {lib.mk_llama_last_error().decode()}")
         if out[0] != 0:
-            result = tuple(out)
-            del _static_scratch_ptrs[device.index]
+            _static_status_pending[device.index] = False   # reported once; the next static launch clears the array
+            if result[0] == 0:
+                result = tuple(out)
     return result
 
 

@@ -453,3 +453,126 @@ class LatencyScheduleBuilder(ScheduleBuilder):
             globs=cls.make_globals(model, skip_attn_reduction=schedule.globs.skip_attn_reduction),
         )
 
+
+
+def check_queues_make_progress(globs: Globals, queues: list[list[Instruction]]) -> None:
+    """Raises ``AssertionError`` if the worker queues cannot all run to their ends.
+
+    Every worker executes its queue strictly in order and an instruction starts only when the
+    counters it waits for have reached their targets, so an assignment that puts an instruction behind
+    one that (transitively) waits for it never finishes - on the device: a wait that runs into its time
+    limit.  The waits are those of the Python VM (``python_vm.py:88-95,110,132,176,255,281-290,353-356``)
+    plus one that only this build's kernel has: when the column-group jobs of a residual projection run
+    each on their own (without ``MK_FLAG_JOINT_RESIDUAL``), the job of the last column group collects the
+    other groups' partial sums of its rows and therefore waits for those jobs.  The assignment policies
+    of ``megakernels_amd/scheduler.py`` keep the linear instruction order within every queue, which
+    satisfies all of it; this check is for hand-made or externally produced queues.
+
+    Targets that the instructions present cannot reach (a schedule that starts in the middle of a
+    layer, its earlier counts already in ``barriers``) count as reached by what is present."""
+    H, KVH = globs.num_attention_heads, globs.num_kv_heads
+    gqa = globs.gqa_ratio()
+    blocks_per_head = globs.qkv_blocks_per_head()
+    real = [[ins for ins in q if ins.opcode() != 0] for q in queues]
+
+    qkv_block_done: dict[tuple[int, int], bool] = {}
+    partial_arrivals: dict[tuple[int, int], int] = {}      # (layer, head group start) -> partitions + merges done
+    partial_present: dict[tuple[int, int], int] = {}
+    row_arrivals: dict[tuple[int, int], int] = {}          # (layer, barrier row 2..5) -> arrivals
+    row_present: dict[tuple[int, int], int] = {}
+    group_job_done: dict[tuple[int, int, int, int], bool] = {}   # (opcode, layer, block, group)
+    lm_dep_layer = globs.num_hidden_layers - 1
+
+    def arrivals_of(ins):
+        """(key, count) pairs this instruction adds when it completes."""
+        op = ins.opcode()
+        if op == 2:
+            if globs.skip_attn_reduction:
+                return [((ins.layer_idx, 2), gqa)]
+            return [((ins.layer_idx, "p", ins.kv_head_idx * gqa), 1)]
+        if op == 3:
+            if ins.is_terminal:
+                return [((ins.layer_idx, 2), globs.attn_reduction_size)]
+            return [((ins.layer_idx, "p", ins.head_start_idx), 1)]
+        if op == 4:
+            return [((ins.layer_idx, 3), ins.end_block_idx - ins.start_block_idx)]
+        if op == 5:
+            return [((ins.layer_idx, 4), len(ins.block_idxs))]
+        if op == 6:
+            return [((ins.layer_idx, 5), ins.end_block_idx - ins.start_block_idx)]
+        return []
+
+    def add(table, key, count):
+        table[key] = table.get(key, 0) + count
+
+    for q in real:
+        for ins in q:
+            op = ins.opcode()
+            if op == 1:
+                for b in ins.block_indices():
+                    qkv_block_done[(ins.layer_idx, b)] = False
+            for key, count in arrivals_of(ins):
+                if len(key) == 3:
+                    add(partial_present, (key[0], key[2]), count)
+                else:
+                    add(row_present, key, count)
+            if op in (4, 6):
+                for b in range(ins.start_block_idx, ins.end_block_idx):
+                    group_job_done[(op, ins.layer_idx, b, ins.reduction_block_idx)] = False
+
+    def reached(table, present, key, target):
+        return table.get(key, 0) >= min(target, present.get(key, 0))
+
+    def ready(ins) -> bool:
+        op = ins.opcode()
+        if op == 1:
+            return ins.layer_idx == 0 or reached(row_arrivals, row_present, (ins.layer_idx - 1, 5), globs.down_proj_total_jobs())
+        if op == 2:
+            heads = list(range(ins.kv_head_idx * gqa, (ins.kv_head_idx + 1) * gqa)) + [H + ins.kv_head_idx, H + KVH + ins.kv_head_idx]
+            return all(qkv_block_done.get((ins.layer_idx, h * blocks_per_head + b), True)
+                       for h in heads for b in range(blocks_per_head))
+        if op == 3:
+            return reached(partial_arrivals, partial_present, (ins.layer_idx, ins.head_start_idx), ins.num_partials)
+        if op in (4, 6):
+            row, target = (2, H) if op == 4 else (4, globs.up_gate_total_blocks())
+            if not reached(row_arrivals, row_present, (ins.layer_idx, row), target):
+                return False
+            groups = globs.o_proj_col_groups() if op == 4 else globs.down_proj_col_groups()
+            if ins.reduction_block_idx == groups - 1:
+                # the collecting job: the other groups' jobs of its rows, where they are scheduled at all
+                return all(group_job_done.get((op, ins.layer_idx, b, g), True)
+                           for b in range(ins.start_block_idx, ins.end_block_idx) for g in range(groups - 1))
+            return True
+        if op == 5:
+            return reached(row_arrivals, row_present, (ins.layer_idx, 3), globs.o_proj_total_jobs())
+        if op == 7:
+            return reached(row_arrivals, row_present, (lm_dep_layer, 5), globs.down_proj_total_jobs())
+        return True
+
+    def complete(ins):
+        op = ins.opcode()
+        if op == 1:
+            for b in ins.block_indices():
+                qkv_block_done[(ins.layer_idx, b)] = True
+        for key, count in arrivals_of(ins):
+            if len(key) == 3:
+                add(partial_arrivals, (key[0], key[2]), count)
+            else:
+                add(row_arrivals, key, count)
+        if op in (4, 6):
+            for b in range(ins.start_block_idx, ins.end_block_idx):
+                group_job_done[(op, ins.layer_idx, b, ins.reduction_block_idx)] = True
+
+    at = [0] * len(real)
+    progressed = True
+    while progressed:
+        progressed = False
+        for w, q in enumerate(real):
+            while at[w] < len(q) and ready(q[at[w]]):
+                complete(q[at[w]])
+                at[w] += 1
+                progressed = True
+    stuck = [(w, q[at[w]]) for w, q in enumerate(real) if at[w] < len(q)]
+    assert not stuck, (
+        f"{len(stuck)} worker queue(s) can never finish: worker {stuck[0][0]} waits at {stuck[0][1]} for instructions "
+        "that are queued behind instructions waiting for it")

@@ -439,3 +439,42 @@ def test_launch_argument_validation():
     with pytest.raises(RuntimeError, match="instructions"):
         interp.interpret(gg)
     gg.instructions = saved
+
+
+def test_diff_test_outfile_dump(tmp_path):
+    """tests/diff_test.py outfile=: the dump the reference's timing tools read
+    (scripts/diff_test.py:231-242) - keys, shapes, and measured events in the reference's slots
+    (include/util.cuh:215-246) in order for the instructions that ran."""
+    import pickle
+    from pathlib import Path
+
+    sys.path.insert(0, str(Path(__file__).resolve().parent))
+    import diff_test
+    from megakernels_amd.scripts import timeline as tl
+
+    out = tmp_path / "timings.pkl"
+    diff_test.main(diff_test.parse(["model=tiny", "prompt_len=20", "ntok=5", "num_attention_partitions=3", f"outfile={out}"]))
+    with open(out, "rb") as f:
+        data = pickle.load(f)   # written a moment ago by this test
+    assert set(data) == {"timings", "timings_native", "instructions", "python_instructions", "cost_per_sm"}
+    workers, slots = data["instructions"].shape[:2]
+    assert workers == 16 and tuple(data["instructions"].shape) == (workers, slots, 32)
+    assert tuple(data["timings"].shape) == (workers, slots, 128) == tuple(data["timings_native"].shape)
+    assert len(data["python_instructions"]) == workers and len(data["cost_per_sm"]) == workers
+    assert all(len(q) <= slots for q in data["python_instructions"])
+    assert all(cost > 0 for cost in data["cost_per_sm"])
+    t = data["timings"].to(torch.int64)
+    ins = data["instructions"]
+    real = ins[:, :, 0] != 0
+    assert int(real.sum()) > 0 and int(t[~real].abs().sum()) == 0
+    # ticks since the launch's first instruction: somebody starts at zero, nothing lasts a second
+    assert int(t[:, :, tl.START][real].min()) == 0 and int(t[real].max()) < 100_000_000
+    assert torch.equal(t[:, :, tl.OPCODE][real], ins[:, :, 0][real].to(torch.int64))
+    matvec = real & (ins[:, :, 0] != 2) & (ins[:, :, 0] != 3) & (t[:, :, tl.FIRST_USE] != 0)
+    assert int(matvec.sum()) > 0
+    chain = (tl.START, tl.AT_GMEM_WAIT, tl.DONE_GMEM_WAIT, tl.LAUNCHER_START, tl.FIRST_USE, tl.LAST_USE, tl.AT_GMEM_STORE, tl.END)
+    for earlier, later in zip(chain, chain[1:]):
+        assert bool((t[:, :, earlier][matvec] <= t[:, :, later][matvec]).all()), (earlier, later)
+    # the stages only the reference has are over when an instruction starts
+    for stage in tl.REFERENCE_ONLY_STAGES:
+        assert torch.equal(t[:, :, stage][real], t[:, :, tl.START][real])

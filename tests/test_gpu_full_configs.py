@@ -105,6 +105,16 @@ def test_c2_full_1b_4096_positions_17_partitions(full_1b):
     _decode(full_1b, prefill=4100, ntok=8, partitions=17)
 
 
+def test_c2_full_1b_64_steps_in_one_launch(full_1b):
+    """The benchmark's own configuration held against the checker for a long launch: 64 decode steps
+    at the full 1B shape, 4096+ cached positions, 17 partitions, without leaving the kernel.  Every
+    step reads, with plain cached loads, K / V rows that earlier steps of the same launch wrote from
+    other compute units, and every step starts behind a grid-wide hand-over of the previous token."""
+    model, model_gpu = full_1b
+    fill_kv_pair(model, model_gpu, upto=4100)
+    _decode(full_1b, prefill=4100, ntok=64, partitions=17)
+
+
 def test_c3_full_1b_16384_positions_24_partitions(full_1b):
     _one_step(full_1b, pos=16390, partitions=24)
     _decode(full_1b, prefill=16390, ntok=4, partitions=24)

@@ -280,3 +280,47 @@ def test_complete_residual_sets_is_what_the_joint_flag_promises():
     only_o = torch.zeros(4, 2, 32, dtype=torch.int32)
     only_o[0, 0, :5] = torch.tensor([4, 0, 0, 1, 0])
     assert shim.complete_residual_sets(only_o, 2048, 8192, 2048)
+
+
+@pytest.mark.parametrize("mode", ["rr", "zz", "wave", "dag"])
+def test_every_assignment_policy_lets_all_queues_finish(mode):
+    """Queues run in order and wait on counters; the job of a residual projection's last column group
+    also waits for the other groups' jobs of its rows when the jobs run on their own.  Every policy
+    keeps the queues free of an instruction stuck behind one that waits for it."""
+    from megakernels_amd.demos.latency.scheduler import check_queues_make_progress
+
+    for cfg, workers, kw in ((cfg_1b(2), 132, {}), (cfg_1b(2), 256, {"num_attention_partitions": 5}),
+                             (LlamaConfig(hidden_size=4096, intermediate_size=14336, num_hidden_layers=2, num_attention_heads=32,
+                                          num_key_value_heads=8, head_dim=128, vocab_size=4096), 256, {"num_attention_partitions": 30})):
+        sched = build(cfg, workers, **kw)
+        check_queues_make_progress(sched.globs, assign_to_sms(mode, schedule=sched))
+
+
+def test_a_queue_order_that_cannot_finish_is_reported():
+    from megakernels_amd.demos.latency.scheduler import check_queues_make_progress
+
+    sched = build(cfg_1b(1), 64)
+    queues = assign_to_sms("rr", schedule=sched)
+    check_queues_make_progress(sched.globs, queues)
+    # put the collecting job (last column group) of some rows in front of the job of another group
+    # of the same rows, on one worker: it waits for a job that is queued behind it
+    jobs = {}
+    for w, q in enumerate(queues):
+        for s, ins in enumerate(q):
+            if isinstance(ins, DownProjResidual):
+                jobs[(ins.start_block_idx, ins.reduction_block_idx)] = (w, s)
+    block = next(b for (b, g) in jobs if g == 3 and (b, 0) in jobs)
+    (wa, sa), (wb, sb) = jobs[(block, 3)], jobs[(block, 0)]
+    collector, other = queues[wa][sa], queues[wb][sb]
+    del queues[wb][sb]
+    queues[wa].insert(sa + 1, other)
+    with pytest.raises(AssertionError, match="can never finish"):
+        check_queues_make_progress(sched.globs, queues)
+    # an instruction in front of the producer of its own input: the same
+    sched = build(cfg_1b(1), 64)
+    queues = assign_to_sms("rr", schedule=sched)
+    w = next(w for w, q in enumerate(queues) if any(isinstance(i, LayerNormDoubleMatVecSiLU) for i in q))
+    s = next(s for s, i in enumerate(queues[w]) if isinstance(i, LayerNormDoubleMatVecSiLU))
+    queues[w].insert(0, queues[w].pop(s))
+    with pytest.raises(AssertionError, match="can never finish"):
+        check_queues_make_progress(sched.globs, queues)
