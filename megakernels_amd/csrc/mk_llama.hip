@@ -128,6 +128,9 @@ constexpr int rows_in_flight(int wanted) { return KC <= 4 ? wanted : (wanted < M
 #ifndef MK_PARK_ALL
 #define MK_PARK_ALL 0               // 1: also the workers that come to O-proj + up/gate from attention park rows
 #endif
+#ifndef MK_RUN_JOBS
+#define MK_RUN_JOBS 1               // consecutive jointly executed jobs of the same blocks run as one
+#endif
 #ifndef MK_POLL_SLEEP
 #define MK_POLL_SLEEP 10            // units of 64 clocks between two looks at a dependency
 #endif
@@ -198,7 +201,8 @@ struct Consts {
 struct alignas(16) SlotDesc {
     uint64_t w0_base;               // buffer the rows are addressed in
     long long gate_delta;           // opcode 5: byte distance from the up matrix to the gate matrix;
-                                    // opcodes 4, 6: column groups executed jointly (0: own group only)
+                                    // opcodes 4, 6: joint execution (0: own group only): the number of column groups
+                                    // G in bits 0-7, the jobs of the block run in one go (1, 2 or 4) in bits 8-15
     uint32_t w0_bytes, row_bytes;
     int ntasks, first_row;
 };
@@ -988,6 +992,13 @@ struct MatvecDesc {
 // are those of the instruction-by-instruction execution.  Task t of such a job: block t / 16, row
 // (t % 16) / G of the job's rows, column group t % G; a wave's tasks (t = wave mod 8) all have column
 // group wave % G, so the wave keeps that group's slice of the activation vector in registers.
+//
+// A worker often holds several of a block's G jobs one after the other in its queue (round-robin
+// assignment of a model with G = 2 gives it both).  Jointly executed they are one piece of work - rows
+// [c * 16 / G, (c + n) * 16 / G) of the block for the n jobs from group c on - with one dependency, one
+// activation vector and one epilogue: the first of the run executes all of them (n = 1, 2 or 4) and
+// signals n arrivals per block, and the others become no-ops when the queue window is decoded.
+constexpr int kAbsorbed = -2;  // SlotDesc::ntasks of a job that an earlier job of its block executes
 __host__ __device__ constexpr bool joint_groups(uint32_t flags, int G, int in_dim) {
     return (flags & MK_FLAG_JOINT_RESIDUAL) != 0 && G > 1 && 16 % G == 0 && G <= 4 &&
            (size_t)in_dim * 2 <= sizeof(Smem::scores);
@@ -1030,7 +1041,31 @@ __device__ __forceinline__ void decode_matvec(SmemPtr sm, int slot, ArgsRef a) {
                     d.first_row = start * 16 + group * (16 / G);
                     d.w0_base = (uint64_t)(uintptr_t)matrix;
                     d.w0_bytes = (uint32_t)((size_t)hid * in_dim * 2);
-                    d.gate_delta = G;
+                    // The run of jobs of the same blocks, with consecutive groups, that this one is part of:
+                    // slots [lo, hi).  It executes in pieces of 4, 2 or 1 jobs from its start; the first
+                    // job of a piece does the work.  (Timing records are kept per instruction: none of this
+                    // in a launch that takes them.)
+                    auto follows = [&](int s) {  // is slot s the job after slot s - 1's?
+                        const InsPtr p = sm->queue[s - 1], q = sm->queue[s];
+                        return q[0] == p[0] && q[1] == p[1] && q[2] == p[2] && q[3] == p[3] && q[4] == p[4] + 1 && q[4] < G;
+                    };
+                    int run = 1;
+                    if (!(a.flags & MK_FLAG_TIMINGS) && end > start && MK_RUN_JOBS) {
+                        const int count = sm->window_count;
+                        int lo = slot, hi = slot + 1;
+                        while (lo > 0 && slot - lo < G && follows(lo)) lo--;
+                        while (hi < count && hi - lo < G && follows(hi)) hi++;
+                        for (int at = lo; at < hi;) {
+                            // (what a piece computes must fit the result buffer)
+                            const int left = hi - at, room = kOutRows / ((end - start) * 16);
+                            const int piece = left >= 4 && room >= 4 ? 4 : left >= 2 && room >= 2 ? 2 : 1;
+                            if (slot == at) run = piece;
+                            else if (slot > at && slot < at + piece) run = 0;
+                            at += piece;
+                        }
+                    }
+                    d.gate_delta = G | (run << 8);
+                    d.ntasks = run ? d.ntasks * run : kAbsorbed;
                 } else {
                     d.first_row = start * 16;
                     // the buffer starts at this column group's first element of the layer's matrix
@@ -1131,9 +1166,11 @@ __device__ __forceinline__ RowRef matvec_row(const MatvecDesc &d, int t) {
         return RowRef{w, (uint32_t)(blk * 16 + (t & 15)) * d.row_bytes};
     }
     if (d.gate_delta > 0) {
-        // jointly executed column-group job: G is a power of two
-        const int G = (int)d.gate_delta, shift = __builtin_ctz((unsigned)G);
-        const int row = d.first_row + (t >> 4) * 16 + ((t & 15) >> shift);
+        // jointly executed column-group jobs: G and the number of jobs are powers of two; a block is
+        // 16 tasks per job
+        const int G = (int)d.gate_delta & 0xff, shift = __builtin_ctz((unsigned)G);
+        const int per_block = (int)(d.gate_delta >> 8) * 16, block_shift = __builtin_ctz((unsigned)per_block);
+        const int row = d.first_row + (t >> block_shift) * 16 + ((t & (per_block - 1)) >> shift);
         return RowRef{d.w0, (uint32_t)row * d.row_bytes + (uint32_t)(t & (G - 1)) * (d.row_bytes >> shift)};
     }
     return RowRef{d.w0, (uint32_t)(d.first_row + t) * d.row_bytes};
@@ -1283,23 +1320,25 @@ __device__ __forceinline__ bool control_matvec_add(const Ctx &c) {
     const int ngroups = in_dim / R;
     const int nblk = end > start ? end - start : 0;
     // column groups executed jointly by this job (0: its own group only), as decoded
-    const int joint = uni((int)((const MK_LDS uint32_t *)&c.sm->desc[c.slot])[2]);
+    const int joint_word = uni((int)((const MK_LDS uint32_t *)&c.sm->desc[c.slot])[2]);
+    const int joint = joint_word & 0xff;                  // G in joint execution, else 0
+    const int run = joint ? joint_word >> 8 : 1;          // jobs of each block that this one executes
     const uint16_t *vec = (is_down ? a.silu_out : a.attn_out) + (joint ? 0 : (size_t)group * R);
     const SyncInfo sy = sync_info(c);
     uint16_t *resid = a.hidden_states;
     // One lane per pair of adjacent residual rows.  Alone, a job owns all 16 rows of its blocks; in
     // joint execution it owns 16 / G rows of each, starting at row group * 16 / G.
-    const int rows_per_block = joint ? 16 / joint : 16;
+    const int rows_per_block = joint ? run * 16 / joint : 16;
     const int pairs_per_block = rows_per_block / 2;
     const int npairs = nblk * pairs_per_block;
     auto row0_of = [&](int p) {
         const int bi = p / pairs_per_block, rp = p % pairs_per_block;
-        return (start + bi) * 16 + (joint ? group * rows_per_block : 0) + rp * 2;
+        return (start + bi) * 16 + (joint ? group * (16 / joint) : 0) + rp * 2;
     };
     // index in sm->out of the first partial sum of the pair's first row (joint: G sums per row, adjacent)
     auto out0_of = [&](int p) {
         const int bi = p / pairs_per_block, rp = p % pairs_per_block;
-        return joint ? bi * 16 + rp * 2 * joint : p * 2;
+        return joint ? bi * 16 * run + rp * 2 * joint : p * 2;
     };
     // The residual rows this instruction updates were last written before its dependency was
     // satisfied, so the controller can fetch them while the consumers work.
@@ -1420,7 +1459,7 @@ __device__ __forceinline__ bool control_matvec_add(const Ctx &c) {
             trace_store_issue(c);
             if (guards_data) wait_stores();
             trace_store_done(c);
-            signal_sharded(c, sy, nblk);
+            signal_sharded(c, sy, nblk * run);
             trace_signalled(c);
         });
 }
@@ -1537,7 +1576,7 @@ constexpr bool kJointSlicePerTask = kConsumerWaves % 4 != 0;
 template <int KC>
 __device__ __forceinline__ const MK_LDS uint32_t *x_source(const Ctx &c, const MatvecDesc &d, int task) {
     if ((d.opcode == 4 || d.opcode == 6) && d.gate_delta > 0)
-        return (const MK_LDS uint32_t *)&c.sm->scores[0][0] + (task & ((int)d.gate_delta - 1)) * (KC * 256);
+        return (const MK_LDS uint32_t *)&c.sm->scores[0][0] + (task & (((int)d.gate_delta & 0xff) - 1)) * (KC * 256);
     return (const MK_LDS uint32_t *)c.sm->x;
 }
 
@@ -2367,6 +2406,12 @@ static __device__ __noinline__ void fetch_window(SmemPtr sm, int base) {
         const int opcode = sm->queue[slot][0];
         if (opcode == 1 || (opcode >= 4 && opcode <= 6)) decode_matvec(sm, slot, a);
         if (opcode == 1 || (opcode >= 4 && opcode <= 7)) decode_sync(sm, slot, a);
+    }
+    wg_barrier();
+    // the jobs that an earlier job of their block executes become no-ops
+    for (int slot = tid; slot < count; slot += kThreads) {
+        const int opcode = sm->queue[slot][0];
+        if ((opcode == 4 || opcode == 6) && sm->desc[slot].ntasks == kAbsorbed) sm->queue[slot][0] = 0;
     }
     wg_barrier();
 }

@@ -107,6 +107,49 @@ def test_column_group_jobs_alone_and_jointly(shape):
         mk_mod.joint_residual_default = None
 
 
+def test_jobs_of_one_block_in_a_row_run_as_one():
+    """A worker that holds several column-group jobs of the same blocks one after the other executes
+    them in one go (pieces of 4, 2 or 1 jobs).  The 1B shape has 4 down-projection groups; the queues
+    are rearranged so that workers hold groups (0, 1, 2, 3), (1, 2, 3), (2, 3), (0, 1) in a row, in
+    falling order (1, 0) - which is no run - and single jobs.  Results and barrier counts are the checker's."""
+    from megakernels_amd.demos.latency.instructions import DownProjResidual
+    from megakernels_amd.scheduler import assign_to_sms, tensorize_instructions
+    from oracle import pyvm
+
+    cfg, workers, pos = config_1b_slice(), 256, 45
+    print(f"case rearranged down-projection jobs hidden={cfg.hidden_size} workers={workers} pos={pos}", flush=True)
+    model = make_model(cfg, max_len=256, seed=0)
+    fill_kv(model, upto=pos)
+    schedule = build_schedule(model, workers)
+    g = schedule.globs
+    queues = assign_to_sms("rr", schedule=schedule)
+    for layer in range(cfg.num_hidden_layers):
+        jobs = {}
+        for queue in queues:
+            for ins in [i for i in queue if isinstance(i, DownProjResidual) and i.layer_idx == layer]:
+                jobs[(ins.start_block_idx, ins.end_block_idx, ins.reduction_block_idx)] = ins
+                queue.remove(ins)
+        ranges = sorted({key[:2] for key in jobs})
+        assert all((*r, grp) in jobs for r in ranges for grp in range(4)), "complete sets of 4 column groups"
+        patterns = [[(0, 1, 2, 3)], [(1, 2, 3), (0,)], [(1, 0), (2, 3)], [(0, 1), (3, 2)]]
+        worker = 0
+        for n, r in enumerate(ranges):
+            for groups in patterns[n % 4]:
+                # the layer's other instructions come first in every queue: down is a layer's last op
+                at = max((k + 1 for k, i in enumerate(queues[worker]) if getattr(i, "layer_idx", -1) == layer), default=0)
+                queues[worker][at:at] = [jobs[(*r, grp)] for grp in groups]
+                worker = (worker + 1) % workers
+    tensorize_instructions(g, queues)
+    gen = torch.Generator().manual_seed(11)
+    g.hidden_states.copy_(torch.randn(cfg.hidden_size, generator=gen).to(torch.bfloat16))
+    g.pos_id = pos
+    model_gpu, schedule_gpu = mirror_to_gpu(model, schedule)
+    pyvm.interpret(g, schedule.get_linear_instructions())
+    _gpu_step(schedule_gpu)
+    report = mismatches(g, schedule_gpu.globs)
+    assert not report, f"tensors differ from the checker: {report}"
+
+
 def _suffix_case(cfg, workers, pos, start_after_op, partitions=1):
     """The reference's diff_test `start_after_op` (scripts/diff_test.py:122-152,198-208): the first part
     of a layer is run by the checker on both sets of buffers, the megakernel then gets only the
