@@ -110,6 +110,21 @@ constexpr int kEpochSlot = 10;      // workspace int: decode steps completed sin
 #ifndef MK_PF_LMHEAD
 #define MK_PF_LMHEAD 2
 #endif
+#ifndef MK_PF_WIDE_OPROJ
+#define MK_PF_WIDE_OPROJ 4
+#endif
+#ifndef MK_PF_WIDE_DOWN
+#define MK_PF_WIDE_DOWN 6
+#endif
+#ifndef MK_WIDE_PARK_QKV
+#define MK_WIDE_PARK_QKV 1
+#endif
+#ifndef MK_WIDE_PARK_UPGATE
+#define MK_WIDE_PARK_UPGATE 1
+#endif
+#ifndef MK_WIDE_PARK_DOWN
+#define MK_WIDE_PARK_DOWN 2
+#endif
 #ifndef MK_PF_WIDE_CAP
 #define MK_PF_WIDE_CAP 2
 #endif
@@ -1546,7 +1561,10 @@ __device__ __forceinline__ void request_rows(const Ctx &c, uint4 (&pool)[NBUF][K
 template <int KC, int J = 0>
 __device__ __forceinline__ void park_chunks(__amdgpu_buffer_rsrc_t rsrc, MK_LDS unsigned char *dst, uint32_t off) {
     if constexpr (J < KC) {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (MK_LDS void *)dst, 16, off, 0, J * 1024, MK_STREAM_AUX);
+        // The instruction's own offset - which moves the place in memory and the place in LDS alike - has 12
+        // bits: whole groups of four chunks go into the scalar offset and the LDS base instead.
+        constexpr int kFar = (J / 4) * 4096;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (MK_LDS void *)(dst + kFar), 16, off, kFar, (J % 4) * 1024, MK_STREAM_AUX);
         park_chunks<KC, J + 1>(rsrc, dst, off);
     }
 }
@@ -1582,7 +1600,7 @@ __device__ __forceinline__ const MK_LDS uint32_t *x_source(const Ctx &c, const M
 
 template <int KC, class Map, int NBUF, int PARKED = 0>
 __device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&pool)[NBUF][KC], const MatvecDesc &d, int mine,
-                                             MK_LDS const unsigned char *slice = nullptr) {
+                                             MK_LDS const unsigned char *slice = nullptr, int parked_rows = PARKED) {
     constexpr int PF = Map::size;
     if (!barrier_inputs_ready(c, true)) return false;
     XPairs<KC> x;
@@ -1595,7 +1613,7 @@ __device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&pool)[NBUF][K
         const float y = mkm::round_bf16(dot_row<KC>(src, x));
         if (c.lane == 0) c.sm->out[task] = y;
     };
-    const int parked_first = mine > PARKED ? mine - PARKED : 0;  // rows from here on are in LDS
+    const int parked_first = mine > parked_rows ? mine - parked_rows : 0;  // rows from here on are in LDS
     const int streamed = PARKED > 0 ? parked_first : mine;
     int base = 0;
     // rounds that are followed by more rows: every row of the round exists, every buffer is refilled
@@ -1667,9 +1685,15 @@ template <> struct FirstBuffers<6> { typedef BufMap<0, 1, 2, 3, 4, 5> type; };
 enum { kConsumerRole = 0, kControllerRole = 1 };
 
 // One matvec instruction (opcode OP, row width KC chunks).
-template <bool TR, int OP, int KC, int PARKED, int ROLE>
+// PARKED > 0: the wave's last PARKED rows come from LDS.  SELF false: an earlier instruction's handler
+// requested them (into the region behind the attention score buffer); SELF true: the instruction
+// requests them itself on entry, into the score buffer, after the rows that go to registers - more
+// rows are then on their way, or there, when the dependency resolves, at no cost in registers.
+template <bool TR, int OP, int KC, int PARKED, int ROLE, int ROWS = 0, bool SELF = false>
 __device__ __forceinline__ bool matvec_impl(SmemPtr lds, int slot, int *refusal) {
-    constexpr int PF = rows_in_flight<KC>(pf_of(OP));
+    static_assert(!SELF || (size_t)kConsumerWaves * PARKED * KC * 1024 <= sizeof(Smem::scores) + sizeof(Smem::park),
+                  "self-parked rows live in the score buffer and the region behind it (which a model with full-width rows only does not use otherwise)");
+    constexpr int PF = ROWS ? ROWS : rows_in_flight<KC>(pf_of(OP));  // rows in flight per wave
     typedef typename FirstBuffers<PF>::type Map;
     const Ctx c = make_ctx<TR>(lds, slot, OP);
     MatvecDesc d;
@@ -1679,14 +1703,19 @@ __device__ __forceinline__ bool matvec_impl(SmemPtr lds, int slot, int *refusal)
     uint4 pool[PF][KC];
     wg_barrier();  // entry: the controller's first requests are out
     trace_first_load(c);
-    request_rows<KC, Map>(c, pool, d, 0, mine > PARKED ? mine - PARKED : 0);
-    const bool ok = consumer_run<KC, Map, PF, PARKED>(
-        c, pool, d, mine, (MK_LDS const unsigned char *)&lds->scores[0][0] + kParkDownOffset + c.wave * (PARKED * KC * 1024));
+    // (a jointly executed job keeps its activation vector in the score buffer: no rows of its own there)
+    const int parked = SELF && (OP == 4 || OP == 6) && d.gate_delta > 0 ? 0 : PARKED;
+    request_rows<KC, Map>(c, pool, d, 0, mine > parked ? mine - parked : 0);
+    MK_LDS unsigned char *slice = (MK_LDS unsigned char *)&lds->scores[0][0] + (SELF ? 0 : kParkDownOffset) + c.wave * (PARKED * KC * 1024);
+    if constexpr (SELF && PARKED > 0) {
+        if (parked > 0) park_rows<KC, PARKED>(c, slice, d, mine > parked ? mine - parked : 0, mine, true);
+    }
+    const bool ok = consumer_run<KC, Map, PF, PARKED>(c, pool, d, mine, slice, parked);
     return ok;
 }
-template <bool TR, int OP, int KC, int PARKED = 0>
+template <bool TR, int OP, int KC, int PARKED = 0, int ROWS = 0, bool SELF = false>
 static __device__ __noinline__ bool op_matvec(SmemPtr lds, int slot, int *refusal) {
-    return matvec_impl<TR, OP, KC, PARKED, kConsumerRole>(lds, slot, refusal);
+    return matvec_impl<TR, OP, KC, PARKED, kConsumerRole, ROWS, SELF>(lds, slot, refusal);
 }
 
 // O-proj followed directly by up/gate, as one handler.  O-proj is short (two rows per wave in the
@@ -2642,6 +2671,10 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
     // handlers that only this kernel calls.
     int refusal = 0;
     const bool controller = uni(tid) >= kConsumerThreads;
+    // A model whose residual projections take several column groups of the hidden width (8B: 4096 = 2 x 2048)
+    // streams in phases that the memory system bounds, not the chain of hand-overs: its narrow rows (one
+    // column group: half the registers of a full-width row) then pay to have more of them in flight.
+    constexpr bool kWide = KC_HID != KC_RED;
     for (int step = 0; step < steps; step++) {
         bool stop = bad_token;
         const int num_slots = uni(sm->args.num_slots);
@@ -2665,7 +2698,7 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
                 if (controller) {
                     ok = uni((int)controller_step<TR, KC_HID, KC_RED, D>(sm, slot, opcode, &refusal)) != 0;
                 } else switch (opcode) {
-                case 1: ok = uni((int)op_matvec<TR, 1, KC_HID>(sm, slot, &refusal)) != 0; break;
+                case 1: ok = uni((int)op_matvec<TR, 1, KC_HID, kWide ? MK_WIDE_PARK_QKV : 0, 0, kWide>(sm, slot, &refusal)) != 0; break;
                 case 2: ok = uni((int)op_attention<TR, D>(sm, slot, &refusal)) != 0; break;
                 case 3: ok = uni((int)op_attention_reduction<TR, D>(sm, slot, &refusal)) != 0; break;
                 case 4:
@@ -2686,9 +2719,9 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
                             break;
                         }
                     }
-                    ok = uni((int)op_matvec<TR, 4, KC_RED>(sm, slot, &refusal)) != 0;
+                    ok = uni((int)op_matvec<TR, 4, KC_RED, 0, kWide ? MK_PF_WIDE_OPROJ : 0>(sm, slot, &refusal)) != 0;
                     break;
-                case 5: ok = uni((int)op_matvec<TR, 5, KC_HID>(sm, slot, &refusal)) != 0; break;
+                case 5: ok = uni((int)op_matvec<TR, 5, KC_HID, kWide ? MK_WIDE_PARK_UPGATE : 0, 0, kWide>(sm, slot, &refusal)) != 0; break;
                 case 6:
                     if constexpr (KC_HID == KC_RED && MK_PAIR_OPROJ_UPGATE && kParkedDownRows > 0) {
                         if (uni(sm->parked_slot) == slot) {
@@ -2696,7 +2729,7 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
                             break;
                         }
                     }
-                    ok = uni((int)op_matvec<TR, 6, KC_RED>(sm, slot, &refusal)) != 0;
+                    ok = uni((int)op_matvec<TR, 6, KC_RED, kWide ? MK_WIDE_PARK_DOWN : 0, kWide ? MK_PF_WIDE_DOWN : 0, kWide>(sm, slot, &refusal)) != 0;
                     break;
                 case 7: ok = uni((int)op_lm_head<TR, KC_HID>(sm, slot, &refusal)) != 0; break;
                 default: ok = bail(make_ctx<TR>(sm, slot, opcode), MK_STATUS_BAD_OPCODE, &refusal);  // reference: trap, include/util.cuh:38
