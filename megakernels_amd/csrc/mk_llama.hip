@@ -125,6 +125,9 @@ constexpr int kEpochSlot = 10;      // workspace int: decode steps completed sin
 #ifndef MK_WIDE_PARK_DOWN
 #define MK_WIDE_PARK_DOWN 2
 #endif
+#ifndef MK_WIDE_AHEAD
+#define MK_WIDE_AHEAD 1             // such a model's O-proj parks the last row per wave of the up/gate instruction behind it
+#endif
 #ifndef MK_PF_WIDE_CAP
 #define MK_PF_WIDE_CAP 2
 #endif
@@ -1689,9 +1692,18 @@ enum { kConsumerRole = 0, kControllerRole = 1 };
 // requested them (into the region behind the attention score buffer); SELF true: the instruction
 // requests them itself on entry, into the score buffer, after the rows that go to registers - more
 // rows are then on their way, or there, when the dependency resolves, at no cost in registers.
-template <bool TR, int OP, int KC, int PARKED, int ROLE, int ROWS = 0, bool SELF = false>
+// AHEAD > 0 (an O projection): the instruction also parks the last row per wave of the up/gate
+// instruction that follows it in the queue, whose rows are AHEAD chunks wide - the O projection waits
+// for attention with little to fetch, and memory is idle meanwhile.  (Requesting that instruction's
+// first rows into registers as well, as the narrow model's pair handler does, was built and measured:
+// 12 % slower - the O projection's own short requests then queue behind 192 KB of rows per CU.)
+// Self-parked up/gate rows start kAheadOffset into the score buffer, behind the vector of a jointly
+// executed O projection.
+constexpr int kAheadOffset = 8192;
+template <bool TR, int OP, int KC, int PARKED, int ROLE, int ROWS = 0, bool SELF = false, int AHEAD = 0>
 __device__ __forceinline__ bool matvec_impl(SmemPtr lds, int slot, int *refusal) {
-    static_assert(!SELF || (size_t)kConsumerWaves * PARKED * KC * 1024 <= sizeof(Smem::scores) + sizeof(Smem::park),
+    constexpr int kSelfOffset = SELF && OP == 5 ? kAheadOffset : 0;
+    static_assert(!SELF || kSelfOffset + (size_t)kConsumerWaves * PARKED * KC * 1024 <= sizeof(Smem::scores) + sizeof(Smem::park),
                   "self-parked rows live in the score buffer and the region behind it (which a model with full-width rows only does not use otherwise)");
     constexpr int PF = ROWS ? ROWS : rows_in_flight<KC>(pf_of(OP));  // rows in flight per wave
     typedef typename FirstBuffers<PF>::type Map;
@@ -1706,16 +1718,36 @@ __device__ __forceinline__ bool matvec_impl(SmemPtr lds, int slot, int *refusal)
     // (a jointly executed job keeps its activation vector in the score buffer: no rows of its own there)
     const int parked = SELF && (OP == 4 || OP == 6) && d.gate_delta > 0 ? 0 : PARKED;
     request_rows<KC, Map>(c, pool, d, 0, mine > parked ? mine - parked : 0);
-    MK_LDS unsigned char *slice = (MK_LDS unsigned char *)&lds->scores[0][0] + (SELF ? 0 : kParkDownOffset) + c.wave * (PARKED * KC * 1024);
+    MK_LDS unsigned char *slice =
+        (MK_LDS unsigned char *)&lds->scores[0][0] + (SELF ? kSelfOffset : kParkDownOffset) + c.wave * (PARKED * KC * 1024);
     if constexpr (SELF && PARKED > 0) {
-        if (parked > 0) park_rows<KC, PARKED>(c, slice, d, mine > parked ? mine - parked : 0, mine, true);
+        // (an up/gate instruction's row may be there already: the O projection before it saw to that)
+        const bool ahead = OP == 5 && uni(lds->parked_slot) == slot;
+        if (parked > 0 && !ahead) park_rows<KC, PARKED>(c, slice, d, mine > parked ? mine - parked : 0, mine, true);
+    }
+    if constexpr (AHEAD > 0) {
+        static_assert(OP == 4 && (size_t)KC * 2048 <= kAheadOffset && MK_WIDE_PARK_UPGATE == 1, "one up/gate row per wave, behind the O projection's vector");
+        // the next instruction of the queue that is not a no-op
+        int next = slot + 1;
+        const int count = uni(lds->window_count);
+        while (next < count && uni(lds->queue[next][0]) == 0) next++;
+        MatvecDesc du;
+        if (next < count && uni(lds->queue[next][0]) == 5 && describe_matvec(lds, next, 5, du)) {
+            const int mine_u = rows_of_wave(du.ntasks, c.wave);
+            MK_LDS unsigned char *slice_u = (MK_LDS unsigned char *)&lds->scores[0][0] + kAheadOffset + c.wave * (AHEAD * 1024);
+            park_rows<AHEAD, 1>(c, slice_u, du, mine_u > 1 ? mine_u - 1 : 0, mine_u, true);
+            if (c.tid == 0) lds->parked_slot = next;
+        }
     }
     const bool ok = consumer_run<KC, Map, PF, PARKED>(c, pool, d, mine, slice, parked);
+    if constexpr (SELF && OP == 5) {
+        if (c.tid == 0) lds->parked_slot = -1;  // (the same slot comes round again in the next step of the launch)
+    }
     return ok;
 }
-template <bool TR, int OP, int KC, int PARKED = 0, int ROWS = 0, bool SELF = false>
+template <bool TR, int OP, int KC, int PARKED = 0, int ROWS = 0, bool SELF = false, int AHEAD = 0>
 static __device__ __noinline__ bool op_matvec(SmemPtr lds, int slot, int *refusal) {
-    return matvec_impl<TR, OP, KC, PARKED, kConsumerRole, ROWS, SELF>(lds, slot, refusal);
+    return matvec_impl<TR, OP, KC, PARKED, kConsumerRole, ROWS, SELF, AHEAD>(lds, slot, refusal);
 }
 
 // O-proj followed directly by up/gate, as one handler.  O-proj is short (two rows per wave in the
@@ -2719,7 +2751,7 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
                             break;
                         }
                     }
-                    ok = uni((int)op_matvec<TR, 4, KC_RED, 0, kWide ? MK_PF_WIDE_OPROJ : 0>(sm, slot, &refusal)) != 0;
+                    ok = uni((int)op_matvec<TR, 4, KC_RED, 0, kWide ? MK_PF_WIDE_OPROJ : 0, false, kWide && MK_WIDE_AHEAD ? KC_HID : 0>(sm, slot, &refusal)) != 0;
                     break;
                 case 5: ok = uni((int)op_matvec<TR, 5, KC_HID, kWide ? MK_WIDE_PARK_UPGATE : 0, 0, kWide>(sm, slot, &refusal)) != 0; break;
                 case 6:
