@@ -80,6 +80,7 @@ constexpr int kHotRows = 4;         // barrier rows 2..5 are sharded
 constexpr int kOutRows = 2048;      // rows staged in LDS between matvec and epilogue
 constexpr int kMaxK = 4096;         // longest activation vector handed through LDS
 constexpr int kScoreCap = 4096;     // tokens per attention partition (LDS score buffer)
+constexpr int kShareLayers = 128;   // layers for which QKV work can be shared between partner workers
 constexpr int kQueueSlots = 192;    // instructions of a worker's queue kept in LDS at a time (a longer queue goes through in windows)
 constexpr int kMaxHeadDim = 128;
 constexpr int kGqa = 4;             // query heads per KV head handled by one attention instruction
@@ -148,6 +149,9 @@ constexpr int rows_in_flight(int wanted) { return KC <= 4 ? wanted : (wanted < M
 #endif
 #ifndef MK_RUN_JOBS
 #define MK_RUN_JOBS 1               // consecutive jointly executed jobs of the same blocks run as one
+#endif
+#ifndef MK_SHARE_QKV
+#define MK_SHARE_QKV 1              // a worker with one QKV block less than its partner takes half of the partner's last block
 #endif
 #ifndef MK_POLL_SLEEP
 #define MK_POLL_SLEEP 10            // units of 64 clocks between two looks at a dependency
@@ -218,7 +222,10 @@ struct Consts {
 // ntasks < 0: the instruction is malformed.
 struct alignas(16) SlotDesc {
     uint64_t w0_base;               // buffer the rows are addressed in
-    long long gate_delta;           // opcode 5: byte distance from the up matrix to the gate matrix;
+    long long gate_delta;           // opcode 1: how the last block is shared with the partner worker (0: it is not):
+                                    // block << 2 | 1 (rows 0-7 of the own last block only) or 2 (also rows 8-15 of the
+                                    // partner's last block);
+                                    // opcode 5: byte distance from the up matrix to the gate matrix;
                                     // opcodes 4, 6: joint execution (0: own group only): the number of column groups
                                     // G in bits 0-7, the jobs of the block run in one go (1, 2 or 4) in bits 8-15
     uint32_t w0_bytes, row_bytes;
@@ -245,6 +252,10 @@ struct Smem {
     Consts k;
     mk_llama_args args;             // the launch arguments, read from here by every instruction
     int flags[16];                  // scratch of the end-of-step reduction
+    // QKV instructions per layer of this worker's queue ([0]) and of its partner's ([1]): how many, and of
+    // the only one: blocks << 20 | its last block
+    int qkv_count[2][kShareLayers];
+    int qkv_info[2][kShareLayers];
     // the matvec instructions' hand-over buffers and attention's share their space: an instruction
     // uses one set or the other, and nothing in them outlives an instruction
     union {
@@ -1016,6 +1027,12 @@ struct MatvecDesc {
 // [c * 16 / G, (c + n) * 16 / G) of the block for the n jobs from group c on - with one dependency, one
 // activation vector and one epilogue: the first of the run executes all of them (n = 1, 2 or 4) and
 // signals n arrivals per block, and the others become no-ops when the queue window is decoded.
+// Models whose residual projections take several column groups of the hidden width (8B) stream their QKV
+// rows in a phase that ends with the workers that hold one block more than the others: those share.
+template <class Args>
+__device__ __forceinline__ bool shares_qkv_blocks(const Args &a) { return MK_SHARE_QKV && a.hidden_size != a.matvec_reduction_size; }
+template <class Args>
+__device__ __forceinline__ int qkv_counter_unit(const Args &a) { return shares_qkv_blocks(a) ? 2 : 1; }
 constexpr int kAbsorbed = -2;  // SlotDesc::ntasks of a job that an earlier job of its block executes
 __host__ __device__ constexpr bool joint_groups(uint32_t flags, int G, int in_dim) {
     return (flags & MK_FLAG_JOINT_RESIDUAL) != 0 && G > 1 && 16 % G == 0 && G <= 4 &&
@@ -1039,7 +1056,22 @@ __device__ __forceinline__ void decode_matvec(SmemPtr sm, int slot, ArgsRef a) {
             const int start = ins[2], end = ins[3];
             const int total_blocks = (a.num_attention_heads + 2 * a.num_kv_heads) * a.head_dim / 16;
             if (start >= 0 && end <= total_blocks && end - start <= kOutRows / 16) {
-                d.ntasks = (end > start ? end - start : 0) * 16;
+                const int nblk = end > start ? end - start : 0;
+                d.ntasks = nblk * 16;
+                // Sharing with the partner worker (share_setup): both have exactly one QKV instruction for
+                // the layer and their block counts differ by one.  The one with more computes rows 0-7 of
+                // its last block only, the other rows 8-15 of that block as well.
+                if (layer < kShareLayers && sm->qkv_count[0][layer] == 1 && sm->qkv_count[1][layer] == 1 &&
+                    (sm->qkv_info[0][layer] >> 20) == nblk) {
+                    const int theirs = sm->qkv_info[1][layer], n_p = theirs >> 20, last_p = theirs & 0xfffff;
+                    if (n_p == nblk + 1 && last_p < total_blocks && nblk * 16 + 8 <= kOutRows) {
+                        d.gate_delta = (last_p << 2) | 2;
+                        d.ntasks += 8;
+                    } else if (n_p == nblk - 1) {
+                        d.gate_delta = ((end - 1) << 2) | 1;
+                        d.ntasks -= 8;
+                    }
+                }
                 d.first_row = start * 16;
                 d.row_bytes = (uint32_t)hid * 2u;
                 d.w0_base = (uint64_t)(uintptr_t)(a.qkv_weights + (size_t)layer * total_blocks * 16 * hid);
@@ -1183,6 +1215,12 @@ __device__ __forceinline__ RowRef matvec_row(const MatvecDesc &d, int t) {
         const WeightBuffer w = {(const uint16_t *)((uintptr_t)d.w0.base + (uintptr_t)shift), d.w0.bytes};
         return RowRef{w, (uint32_t)(blk * 16 + (t & 15)) * d.row_bytes};
     }
+    if (d.opcode == 1) {
+        // the last 8 tasks of a worker that helps its partner: rows 8-15 of the partner's last block
+        const bool helps = ((int)d.gate_delta & 3) == 2 && t >= d.ntasks - 8;
+        const int row = helps ? ((int)d.gate_delta >> 2) * 16 + 8 + (t - (d.ntasks - 8)) : d.first_row + t;
+        return RowRef{d.w0, (uint32_t)row * d.row_bytes};
+    }
     if (d.gate_delta > 0) {
         // jointly executed column-group jobs: G and the number of jobs are powers of two; a block is
         // 16 tasks per job
@@ -1198,7 +1236,9 @@ __device__ __forceinline__ RowRef matvec_row(const MatvecDesc &d, int t) {
 // opcode 1: RMSNorm + QKV matvec + RoPE + KV append  (python_vm.py:168-248;
 // reference device op: demos/low-latency-llama/rms_matvec_rope_append.cu:10-231)
 // ---------------------------------------------------------------------------------------------
-template <int KC>
+// SHARE: the model is of the kind whose workers share QKV blocks (share_setup); its per-head counters
+// count half blocks.
+template <int KC, bool SHARE>
 __device__ __forceinline__ bool control_qkv(const Ctx &c) {
     const InsPtr ins = c.sm->queue[c.slot];
     ArgsRef a = c.sm->args;
@@ -1206,9 +1246,15 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
     const int hid = a.hidden_size, D = a.head_dim, H = a.num_attention_heads, KVH = a.num_kv_heads;
     const int nblk = end > start ? end - start : 0;
     const int k_start = H * D, v_start = k_start + KVH * D;
+    // half a block shared with the partner worker (see decode_matvec): which, and which half
+    const int share = SHARE ? uni((int)((const MK_LDS uint32_t *)&c.sm->desc[c.slot])[2]) : 0;
+    const int share_mode = share & 3, share_block = share >> 2;
+    const int own_rows = nblk * 16 - (share_mode == 1 ? 8 : 0);
+    const int npairs = (own_rows + (share_mode == 2 ? 8 : 0)) / 2;   // one lane per pair of adjacent rows
+    auto row0_of = [&](int p) { return p * 2 < own_rows ? start * 16 + p * 2 : share_block * 16 + 8 + (p * 2 - own_rows); };
     constexpr int kPre = 2;
     float rot[kPre][4] = {{1.0f, 1.0f, 0.0f, 0.0f}, {1.0f, 1.0f, 0.0f, 0.0f}};
-    const bool prefetched = nblk * 8 <= kPre * 64;
+    const bool prefetched = npairs <= kPre * 64;
     PollTicket ticket = {nullptr, 0, 0};
     const SyncInfo sy = sync_info(c);
     uint4 wraw[KC];
@@ -1216,12 +1262,12 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
         c,
         [&]() {
             ticket = poll_issue(c, sy);
-            if (nblk > 0) load_row<KC>(wraw, a.attn_norm_weights + (size_t)layer * hid, c.lane);
+            if (npairs > 0) load_row<KC>(wraw, a.attn_norm_weights + (size_t)layer * hid, c.lane);
         },
         [&](auto release) {
             if (layer > 0 && !poll_wait(c, ticket, true, sy.target, release)) return false;
             trace_event(c, kEvDepReady, MK_TIMING_DONE_GMEM_WAIT);
-            if (nblk > 0) {
+            if (npairs > 0) {
                 // layer 0 of a launch that was given a token reads the embedding row itself; the
                 // worker holding the first block also makes it the residual stream (every later
                 // reader of hidden_states waits, through attention, for this worker's signal)
@@ -1230,7 +1276,7 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
                 uint4 x[KC];
                 load_xq<KC>(x, src, c.lane);
                 release();
-                if (from_table && start == 0) {
+                if (from_table && start == 0 && nblk > 0) {
 #pragma unroll
                     for (int j = 0; j < KC; j++) {
                         uint16_t *dst = a.hidden_states + j * 512 + c.lane * 8;
@@ -1253,8 +1299,8 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
 #pragma unroll
                 for (int k = 0; k < kPre; k++) {
                     const int p = c.lane + k * 64;
-                    const int row0 = start * 16 + p * 2;
-                    if (p < nblk * 8 && row0 < v_start) {
+                    const int row0 = row0_of(p);
+                    if (p < npairs && row0 < v_start) {
                         const int d = row0 % D;
                         const float *cs = a.rope_cos + (size_t)a.pos_id * D + d;
                         const float *sn = a.rope_sin + (size_t)a.pos_id * D + d;
@@ -1270,7 +1316,7 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
             // epilogue: one lane per adjacent row pair
             const size_t kv_row = ((size_t)layer * a.kv_max_len + a.pos_id) * KVH * D;
             auto emit = [&](int p, float c0, float c1, float s0, float s1) {
-                const int row0 = start * 16 + p * 2;
+                const int row0 = row0_of(p);
                 const float y0 = c.sm->out[p * 2], y1 = c.sm->out[p * 2 + 1];
                 uint32_t packed;
                 if (row0 < v_start) {
@@ -1290,10 +1336,10 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
             if (prefetched) {
 #pragma unroll
                 for (int k = 0; k < kPre; k++)
-                    if (c.lane + k * 64 < nblk * 8) emit(c.lane + k * 64, rot[k][0], rot[k][1], rot[k][2], rot[k][3]);
+                    if (c.lane + k * 64 < npairs) emit(c.lane + k * 64, rot[k][0], rot[k][1], rot[k][2], rot[k][3]);
             } else {
-                for (int p = c.lane; p < nblk * 8; p += 64) {
-                    const int row0 = start * 16 + p * 2;
+                for (int p = c.lane; p < npairs; p += 64) {
+                    const int row0 = row0_of(p);
                     float c0 = 1.0f, c1 = 1.0f, s0 = 0.0f, s1 = 0.0f;
                     if (row0 < v_start) {
                         const int d = row0 % D;
@@ -1307,8 +1353,13 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
             trace_store_issue(c);
             wait_stores();
             trace_store_done(c);
-            // one arrival per block on its head's counter (python_vm.py:248)
-            for (int b = c.lane; b < nblk; b += 64) add_i32(pad_ptr(c, layer, 0, (start + b) / (D / 16)), 1);
+            // One arrival per block on its head's counter (python_vm.py:248).  Where blocks can be shared the
+            // counters count half blocks while the kernel runs: two for a whole block, one each from the two
+            // workers that share one.
+            for (int b = c.lane; b < nblk + (share_mode == 2 ? 1 : 0); b += 64) {
+                const int block = b < nblk ? start + b : share_block;
+                add_i32(pad_ptr(c, layer, 0, block / (D / 16)), !SHARE || b >= nblk || (share_mode == 1 && b == nblk - 1) ? 1 : 2);
+            }
             trace_signalled(c);
         });
 }
@@ -1657,10 +1708,10 @@ __device__ __forceinline__ bool consumer_run(const Ctx &c, uint4 (&pool)[NBUF][K
     return true;
 }
 
-template <int KC>
+template <int KC, bool WIDE>
 __device__ __forceinline__ bool control_matvec(const Ctx &c) {
     switch (c.opcode) {
-    case 1: return control_qkv<KC>(c);
+    case 1: return control_qkv<KC, WIDE && MK_SHARE_QKV>(c);
     case 4: return control_matvec_add<KC, false>(c);
     case 5: return control_upgate<KC>(c);
     default: return control_matvec_add<KC, true>(c);
@@ -1700,7 +1751,7 @@ enum { kConsumerRole = 0, kControllerRole = 1 };
 // Self-parked up/gate rows start kAheadOffset into the score buffer, behind the vector of a jointly
 // executed O projection.
 constexpr int kAheadOffset = 8192;
-template <bool TR, int OP, int KC, int PARKED, int ROLE, int ROWS = 0, bool SELF = false, int AHEAD = 0>
+template <bool TR, int OP, int KC, int PARKED, int ROLE, int ROWS = 0, bool SELF = false, int AHEAD = 0, bool WIDE = false>
 __device__ __forceinline__ bool matvec_impl(SmemPtr lds, int slot, int *refusal) {
     constexpr int kSelfOffset = SELF && OP == 5 ? kAheadOffset : 0;
     static_assert(!SELF || kSelfOffset + (size_t)kConsumerWaves * PARKED * KC * 1024 <= sizeof(Smem::scores) + sizeof(Smem::park),
@@ -1710,7 +1761,7 @@ __device__ __forceinline__ bool matvec_impl(SmemPtr lds, int slot, int *refusal)
     const Ctx c = make_ctx<TR>(lds, slot, OP);
     MatvecDesc d;
     if (!describe_matvec(lds, slot, OP, d)) return bail(c, MK_STATUS_BAD_INSTRUCTION, refusal);
-    if constexpr (ROLE == kControllerRole) return control_matvec<KC>(c);
+    if constexpr (ROLE == kControllerRole) return control_matvec<KC, WIDE>(c);
     const int mine = rows_of_wave(d.ntasks, c.wave);
     uint4 pool[PF][KC];
     wg_barrier();  // entry: the controller's first requests are out
@@ -2007,8 +2058,11 @@ __device__ __forceinline__ bool attention_impl(SmemPtr lds, int slot, int *refus
         // wait: Q heads, K head and V head of this step are complete (python_vm.py:281-290)
         const int col = c.lane < G ? h0 + c.lane : c.lane == G ? H + kvh : H + KVH + kvh;
         const bool mine = c.lane < G + 2;
-        const bool ok = poll_counters(c, mine ? pad_ptr(c, layer, 0, col) : nullptr, mine ? bar_ptr(c, layer, 0, col) : nullptr,
-                                      false, D / 16);
+        // (where QKV blocks can be shared, the counters count half blocks, `barriers` whole ones)
+        const int unit = qkv_counter_unit(a);
+        PollTicket ticket = poll_issue(c, mine ? pad_ptr(c, layer, 0, col) : nullptr, mine ? bar_ptr(c, layer, 0, col) : nullptr);
+        ticket.base *= unit;
+        const bool ok = poll_wait(c, ticket, false, unit * (D / 16), []() {});
         trace_event(c, kEvDepReady, MK_TIMING_DONE_GMEM_WAIT);
         if (!barrier_inputs_ready(c, ok)) return false;
         trace_event(c, kEvInputReady);
@@ -2427,7 +2481,7 @@ static __device__ __noinline__ bool op_attention_reduction(SmemPtr lds, int slot
 template <bool TR, int KC_HID, int KC_RED, int D>
 __device__ __forceinline__ bool controller_step(SmemPtr sm, int slot, int opcode, int *refusal) {
     switch (opcode) {
-    case 1: return matvec_impl<TR, 1, KC_HID, 0, kControllerRole>(sm, slot, refusal);
+    case 1: return matvec_impl<TR, 1, KC_HID, 0, kControllerRole, 0, false, 0, KC_HID != KC_RED>(sm, slot, refusal);
     case 2: return attention_impl<TR, D, kControllerRole>(sm, slot, refusal);
     case 3: return reduction_impl<TR, D, kControllerRole>(sm, slot, refusal);
     case 4: return matvec_impl<TR, 4, KC_RED, 0, kControllerRole>(sm, slot, refusal);
@@ -2450,6 +2504,39 @@ __device__ __forceinline__ bool controller_step(SmemPtr sm, int slot, int opcode
 // a window of the worker's queue is copied into LDS and its matvec instructions are decoded, so that
 // taking an instruction never waits on HBM.  The usual queue fits the window and is fetched once per
 // launch; a longer one goes through window by window, every step.
+// Which QKV instructions this worker and its partner (the neighbouring worker: w ^ 1) hold, per layer.
+// The reference's schedule deals the 16-row blocks of the QKV projection out evenly up to one block (8B:
+// 384 blocks, two for every other worker, one for the rest), and the phase ends with the workers that
+// have one more, which fetch their last rows after the dependency has resolved.  Where the two partners'
+// instructions of a layer differ by one block, the one with fewer takes rows 8-15 of the other's last
+// block: both decide so on their own, from the same two queues.
+static __device__ __noinline__ void share_setup(SmemPtr sm) {
+    ArgsRef a = sm->args;
+    const int tid = (int)threadIdx.x;
+    MK_LDS int *tables = &sm->qkv_count[0][0];
+    static_assert(offsetof(Smem, qkv_info) == offsetof(Smem, qkv_count) + sizeof(Smem::qkv_count), "cleared as one array");
+    for (int i = tid; i < 4 * kShareLayers; i += kThreads) tables[i] = 0;
+    wg_barrier();
+    const int workers = (int)gridDim.x;
+    if (shares_qkv_blocks(a) && workers % 2 == 0 && a.num_layers <= kShareLayers) {
+        const int partner = (int)blockIdx.x ^ 1;
+        for (int s = tid; s < 2 * a.num_slots; s += kThreads) {
+            const int who = s < a.num_slots ? 0 : 1, slot = who ? s - a.num_slots : s;
+            const MK_GLOBAL int *ins =
+                as_global(a.instructions) + ((size_t)(who ? partner : (int)blockIdx.x) * a.num_slots + slot) * MK_INSTRUCTION_WORDS;
+            if (ins[0] != 1) continue;
+            const int layer = ins[1], start = ins[2], end = ins[3];
+            if (layer < 0 || layer >= a.num_layers) continue;
+            const int nblk = end > start ? end - start : 0;
+            const bool fine = start >= 0 && end < (1 << 20) && nblk <= kOutRows / 16;
+            // (a malformed instruction counts twice: no sharing with it)
+            __hip_atomic_fetch_add(&sm->qkv_count[who][layer], fine ? 1 : 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (fine) sm->qkv_info[who][layer] = (nblk << 20) | (nblk > 0 ? end - 1 : 0);  // (meaningful when it is the only one)
+        }
+    }
+    wg_barrier();
+}
+
 static __device__ __noinline__ void fetch_window(SmemPtr sm, int base) {
     ArgsRef a = sm->args;
     const int tid = (int)threadIdx.x;
@@ -2545,8 +2632,9 @@ static __device__ __noinline__ bool end_of_step(SmemPtr sm, int step, int steps)
                     if (v[u] == 0) continue;
                     st_i32(pads + (size_t)k * kPadInts, 0);
                     const int col = k % pc, lr = k / pc;
+                    // (row 0, the QKV blocks of a head, is counted in half blocks)
                     if (!reset && col < cols)
-                        add_i32(barriers + ((size_t)(lr / 2) * MK_BARRIER_ROWS + lr % 2) * cols + col, v[u]);
+                        add_i32(barriers + ((size_t)(lr / 2) * MK_BARRIER_ROWS + lr % 2) * cols + col, lr % 2 == 0 ? v[u] / qkv_counter_unit(a) : v[u]);
                 }
             }
         }
@@ -2689,6 +2777,7 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
     // a launch that was given a token outside the vocabulary: every workgroup sees the same bad token
     // and skips its queue
     const bool bad_token = a.token_in && uni(sm->token) < 0;
+    share_setup(sm);
     fetch_window(sm, 0);
     if (bad_token && tid == kConsumerThreads) {
         record_status(make_ctx<TR>(sm, 0, 0), MK_STATUS_BAD_TOKEN);

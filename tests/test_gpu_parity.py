@@ -84,6 +84,17 @@ def test_8b_slice_column_groups():
     _one_step_case(config_8b_slice(), workers=256, pos=77)
 
 
+def test_8b_slice_shared_qkv_blocks_under_every_assignment():
+    """On the 4096-wide shape neighbouring workers whose QKV instructions of a layer differ by one block share
+    the larger one's last block (rows 8-15 go to the neighbour).  Who neighbours whom depends on the assignment,
+    and with fewer workers than instructions per layer a worker holds several QKV instructions (no sharing then):
+    results and barrier counts are the checker's in every case."""
+    for sched in ("rr", "zz", "wave", "dag"):
+        _one_step_case(config_8b_slice(layers=2), workers=256, pos=33, sched=sched)
+    _one_step_case(config_8b_slice(layers=2), workers=250, pos=33)   # 384 blocks over 250 workers: other pairings
+    _one_step_case(config_8b_slice(layers=2), workers=100, pos=33)
+
+
 def test_8b_slice_split_kv():
     _one_step_case(config_8b_slice(), workers=256, pos=1500, partitions=8, max_len=2048)
 
