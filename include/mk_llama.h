@@ -186,7 +186,7 @@ int mk_llama_launch(const mk_llama_args *args, void *hip_stream);
  * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No
  * counterpart in the reference.  `args->workspace` and `args->workspace_bytes` are ignored; the
  * workspace is an array inside the library (2 MiB per GPU, held until the process ends), which is
- * enough for every shape the kernel has an instance for (1B: 280 KB, 8B with 32 layers: 1.01 MiB).
+ * enough for every shape the kernel has an instance for (1B: 296 KB, 8B with 32 layers: 1.04 MiB).
  * Shapes that need more are refused with -6 and a message.  The call allocates nothing: it zeroes
  * the part of the array it is going to use with a small kernel on `hip_stream`, then launches as
  * mk_llama_launch does.  `*scratch_out` (may be NULL) receives the array's device address, which is

@@ -153,6 +153,9 @@ constexpr int rows_in_flight(int wanted) { return KC <= 4 ? wanted : (wanted < M
 #ifndef MK_SHARE_QKV
 #define MK_SHARE_QKV 1              // a worker with one QKV block less than its partner takes half of the partner's last block
 #endif
+#ifndef MK_STAGE_QUERY
+#define MK_STAGE_QUERY 1            // attention takes the query and the step's K / V row from their stamped copies
+#endif
 #ifndef MK_POLL_SLEEP
 #define MK_POLL_SLEEP 10            // units of 64 clocks between two looks at a dependency
 #endif
@@ -177,7 +180,7 @@ constexpr int kParkBytes = kParkRegionBytes > kScoreBytes ? kParkRegionBytes - k
 // workspace layout (ints unless noted)
 // ---------------------------------------------------------------------------------------------
 struct WsLayout {
-    size_t status, shards, argmax, partial, pads, total_bytes;
+    size_t status, shards, argmax, partial, pads, stamped, total_bytes;
 };
 constexpr int kMaxWorkers = 1024;   // workers that can report an LM-head maximum
 constexpr int kPadInts = 32;        // a padded counter owns a 128-byte line
@@ -199,6 +202,10 @@ __host__ __device__ inline WsLayout ws_layout(int L, int hid, int inter, int R) 
     // the per-head counters (barrier rows 0 and 1), one cache line each
     off = (off + 31) & ~(size_t)31;
     w.pads = off;     off += (size_t)L * 2 * pad_cols(hid) * kPadInts;
+    // stamped copies of what QKV hands to attention: 8 bytes per bf16 pair (the query, hid / 2 pairs,
+    // then the step's K row and V row, at most hid / 8 pairs each)
+    off = (off + 31) & ~(size_t)31;
+    w.stamped = off;  off += 2 * (size_t)hid;
     w.total_bytes = off * 4;
     return w;
 }
@@ -210,6 +217,7 @@ __host__ __device__ inline WsLayout ws_layout(int L, int hid, int inter, int R) 
 struct Consts {
     int *status, *shards, *argmax, *pads;  // regions of the workspace
     uint64_t *partial;              // residual partial sums as (value, tag) pairs
+    uint64_t *stamped;              // (bf16 pair, stamp) copies of the query and of the step's K and V rows
     uint32_t epoch;                 // decode steps completed in this workspace before the current one
     int *trace_base;                // this worker's rows of `timings`, or nullptr when tracing is off
     long long spin_ticks;           // limit of a dependency wait, in wall-clock ticks
@@ -272,6 +280,12 @@ struct Smem {
     alignas(16) float scores[kScoreCap][kGqa];  // attention: one partition's scores, then probabilities
     alignas(16) unsigned char park[kParkBytes];  // the parked rows' region continues here
     int parked_slot;                               // the down projection whose last rows per wave are parked, or -1
+    // attention: the four query heads and the step's K and V row of the KV head as bf16 pairs, when the
+    // controller took them from their stamped copies (attn_staged != 0)
+    int attn_staged;
+    alignas(16) uint32_t attn_q[kGqa * kMaxHeadDim / 2];
+    alignas(16) uint32_t attn_k[kMaxHeadDim / 2];
+    alignas(16) uint32_t attn_v[kMaxHeadDim / 2];
     alignas(16) SlotDesc desc[kQueueSlots];        // the matvec instructions of the window, decoded
     alignas(16) SyncDesc sync[kQueueSlots];        // ... and where their counters live
     alignas(16) int queue[kQueueSlots][MK_INSTRUCTION_WORDS];  // a window of this worker's instructions
@@ -319,6 +333,7 @@ __device__ __forceinline__ uint4 ld_b128(const void *p) {
     return make_uint4((uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32));
 }
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 // immutable data (rope tables, old KV rows): ordinary cached 16-byte load
 __device__ __forceinline__ uint4 ld_const_b128(const void *p) {
     const u32x4 v = *as_global((const u32x4 *)p);
@@ -520,6 +535,12 @@ __device__ __forceinline__ Ctx make_ctx(SmemPtr sm, int slot, int opcode) {
 __device__ __forceinline__ int *ws_status(const Ctx &c) { return uni(c.sm->k.status); }
 __device__ __forceinline__ int *ws_shards(const Ctx &c) { return uni(c.sm->k.shards); }
 __device__ __forceinline__ uint64_t *ws_partial(const Ctx &c) { return uni(c.sm->k.partial); }
+// stamped copies: the query at pair 0, the K row at pair hidden / 2, the V row behind it
+__device__ __forceinline__ uint64_t *ws_stamped_q(const Ctx &c) { return uni(c.sm->k.stamped); }
+__device__ __forceinline__ uint64_t *ws_stamped_k(const Ctx &c) { return uni(c.sm->k.stamped) + uni(c.sm->args.hidden_size) / 2; }
+__device__ __forceinline__ uint64_t *ws_stamped_v(const Ctx &c) {
+    return ws_stamped_k(c) + uni(c.sm->args.num_kv_heads) * uni(c.sm->args.head_dim) / 2;
+}
 __device__ __forceinline__ long long spin_ticks(const Ctx &c) {
     const long long v = c.sm->k.spin_ticks;
     return ((long long)uni((int)(v >> 32)) << 32) | (uint32_t)uni((int)v);
@@ -670,6 +691,18 @@ __device__ __forceinline__ bool poll_wait(const Ctx &c, PollTicket t, bool sum_m
 }
 __device__ bool poll_counters(const Ctx &c, const int *ptr, const int *in_barriers, bool sum_mode, int target) {
     return poll_wait(c, poll_issue(c, ptr, in_barriers), sum_mode, target, []() {});
+}
+
+// Stamp of what one layer writes in one decode step: differs from whatever an entry held before (an
+// earlier layer or step, or the zero of a fresh workspace).
+__device__ __forceinline__ uint32_t layer_stamp(const Ctx &c, int layer) {
+    const uint32_t step = (uint32_t)uni((int)c.sm->k.epoch);
+    const uint32_t stamp = step * (uint32_t)uni(c.sm->args.num_layers) + (uint32_t)layer + 1u;
+    return stamp ? stamp : 1u;
+}
+// One bf16 pair of a stamped copy: a single 8-byte store, so whoever sees the stamp sees the value.
+__device__ __forceinline__ void st_stamped(uint64_t *vec, int pair, uint32_t value, uint32_t stamp) {
+    st_u64(vec + pair, ((uint64_t)stamp << 32) | value);
 }
 
 // The decoded counters of the instruction in the context's slot, as scalars.
@@ -1257,6 +1290,7 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
     const bool prefetched = npairs <= kPre * 64;
     PollTicket ticket = {nullptr, 0, 0};
     const SyncInfo sy = sync_info(c);
+    const uint32_t stamp = layer_stamp(c, layer);
     uint4 wraw[KC];
     return controller_sequence(
         c,
@@ -1332,6 +1366,8 @@ __device__ __forceinline__ bool control_qkv(const Ctx &c) {
                 else if (row0 < v_start) dst = a.k_cache + kv_row + (row0 - k_start);
                 else dst = a.v_cache + kv_row + (row0 - v_start);
                 st_u32(dst, packed);
+                // and the stamped copy that attention looks for (query | K row | V row: the order of the rows)
+                st_stamped(ws_stamped_q(c), row0 >> 1, packed, stamp);
             };
             if (prefetched) {
 #pragma unroll
@@ -2062,7 +2098,75 @@ __device__ __forceinline__ bool attention_impl(SmemPtr lds, int slot, int *refus
         const int unit = qkv_counter_unit(a);
         PollTicket ticket = poll_issue(c, mine ? pad_ptr(c, layer, 0, col) : nullptr, mine ? bar_ptr(c, layer, 0, col) : nullptr);
         ticket.base *= unit;
-        const bool ok = poll_wait(c, ticket, false, unit * (D / 16), []() {});
+        // The QKV instructions leave what attention needs of this step - the query, and the step's K and
+        // V row for the partition that holds the newest position - twice: in the tensors, followed by an
+        // arrival on the heads' counters once the stores are acknowledged; and as stamped copies in the
+        // workspace (8 bytes per bf16 pair: value, stamp of step and layer), which need neither.  The
+        // controller looks at both.  Usually the copies complete first and ARE the data - one trip to memory
+        // instead of acknowledgement, arrival, look at the counter and fetch - and go to the consumers through
+        // LDS; the counters cover arrivals from before the launch, whose data exists in the tensors only.
+        // (1 to 2 KB that 17 to 32 workers look at; the same for the 4 to 32 KB vectors between the matvec
+        // instructions, which all 256 workers would pull, costs more than it saves.)
+        constexpr int NQ = D / 64;  // 16-byte looks per lane that cover the four heads' query
+        const bool has_new = uni((int)(a.pos_id >= t0 && a.pos_id < t0 + T)) != 0;
+        const bool staging = MK_STAGE_QUERY && H * D == a.hidden_size && KVH * kGqa == H;
+        const uint32_t stamp = layer_stamp(c, layer);
+        const uint64_t *sq = ws_stamped_q(c) + (size_t)h0 * (D / 2) + c.lane * 2;
+        // lanes [0, D/4): two pairs each of the K row; lanes [D/4, D/2): of the V row
+        const bool kv_lane = has_new && c.lane < D / 2;
+        const uint64_t *skv = (c.lane < D / 4 ? ws_stamped_k(c) : ws_stamped_v(c) - D / 2) + (size_t)kvh * (D / 2) + c.lane * 2;
+        uint4 qraw[NQ], kvraw = make_uint4(0, 0, 0, 0);
+        auto look = [&]() {
+#pragma unroll
+            for (int j = 0; j < NQ; j++) qraw[j] = ld_b128(sq + j * 128);
+            if (kv_lane) kvraw = ld_b128(skv);
+        };
+        auto complete = [&]() {
+            bool all = !kv_lane || (kvraw.y == stamp && kvraw.w == stamp);
+#pragma unroll
+            for (int j = 0; j < NQ; j++) all &= qraw[j].y == stamp && qraw[j].w == stamp;
+            return __all(all) != 0;
+        };
+        bool ok = true, staged = false;
+        if (staging) {
+            look();
+            const long long w0 = wall_clock64();
+            const long long limit = spin_ticks(c);
+            const int *status = ws_status(c);
+            int v = ticket.value, st = ticket.status;
+            while (true) {
+                if (complete()) {
+                    staged = true;
+                    break;
+                }
+                if (__all(ticket.ptr == nullptr || v + ticket.base >= unit * (D / 16))) break;
+                if (__any(st != 0)) {
+                    ok = false;
+                    break;
+                }
+                if (wall_clock64() - w0 > limit) {
+                    if (c.lane == 0) record_status(c, MK_STATUS_BARRIER_TIMEOUT);
+                    ok = false;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(MK_POLL_SLEEP);
+                v = ticket.ptr ? ld_i32(ticket.ptr) : 0;
+                st = c.lane == 63 ? ld_i32(status) : 0;
+                look();
+            }
+            compiler_fence();
+        } else {
+            ok = poll_wait(c, ticket, false, unit * (D / 16), []() {});
+        }
+        if (staged) {
+#pragma unroll
+            for (int j = 0; j < NQ; j++) *(MK_LDS u32x2 *)&sm->attn_q[j * 128 + c.lane * 2] = u32x2{qraw[j].x, qraw[j].z};
+            if (kv_lane) {
+                MK_LDS uint32_t *dst = c.lane < D / 4 ? &sm->attn_k[c.lane * 2] : &sm->attn_v[(c.lane - D / 4) * 2];
+                *(MK_LDS u32x2 *)dst = u32x2{kvraw.x, kvraw.z};
+            }
+        }
+        if (c.lane == 0) sm->attn_staged = staged ? 1 : 0;
         trace_event(c, kEvDepReady, MK_TIMING_DONE_GMEM_WAIT);
         if (!barrier_inputs_ready(c, ok)) return false;
         trace_event(c, kEvInputReady);
@@ -2095,10 +2199,19 @@ __device__ __forceinline__ bool attention_impl(SmemPtr lds, int slot, int *refus
     auto token_of = [&](int rd) { return rd * NSLOT + c.wave * TPW + tok_in_wave; };
     // rows older than this step are immutable; the row at pos_id was written by another CU a moment
     // ago and needs a coherent load
+    // (the controller may have found the query and the step's rows as stamped copies: they are in LDS then, and
+    // the tensors' own copies of them are not known to have landed; `staged` is set once the dependency is known)
+    bool staged = false;
+    auto lds_row = [&](const MK_LDS uint32_t *row) {
+        const u32x4 v = *(const MK_LDS u32x4 *)(row + sub * 4);
+        return uint4{v.x, v.y, v.z, v.w};
+    };
+    auto newest_row = [&](const uint16_t *kvb) {
+        return staged ? lds_row(kvb == vbase ? sm->attn_v : sm->attn_k) : ld_b128(kvb + (size_t)a.pos_id * tok_stride);
+    };
     auto load_kv = [&](const uint16_t *kvb, int r) {
         const int t = t0 + r;
-        const uint16_t *p = kvb + (size_t)t * tok_stride;
-        return t == a.pos_id ? ld_b128(p) : ld_const_b128(p);
+        return t == a.pos_id ? newest_row(kvb) : ld_const_b128(kvb + (size_t)t * tok_stride);
     };
 
     // Rounds are processed in batches of RU so that RU row loads are in flight per lane.  The first
@@ -2120,16 +2233,18 @@ __device__ __forceinline__ bool attention_impl(SmemPtr lds, int slot, int *refus
 
     trace_consumer_first_use(c);
     uint4 q[G];  // this lane's 8 dims of the four query heads, as bf16 pairs
+    staged = uni(sm->attn_staged) != 0;
     {
 #pragma unroll
-        for (int h = 0; h < G; h++) q[h] = ld_b128(a.q_post_rope + (size_t)(h0 + h) * D + sub * 8);
+        for (int h = 0; h < G; h++)
+            q[h] = staged ? lds_row(&sm->attn_q[h * (D / 2)]) : ld_b128(a.q_post_rope + (size_t)(h0 + h) * D + sub * 8);
         // the newest token's rows, if they fall into the first batch
 #pragma unroll
         for (int u = 0; u < RU; u++) {
             const int r = token_of(u);
             if (r < T && t0 + r == a.pos_id) {
-                kraw[u] = ld_b128(kbase + (size_t)(t0 + r) * tok_stride);
-                vraw[u] = ld_b128(vbase + (size_t)(t0 + r) * tok_stride);
+                kraw[u] = newest_row(kbase);
+                vraw[u] = newest_row(vbase);
             }
         }
     }
@@ -2171,7 +2286,10 @@ __device__ __forceinline__ bool attention_impl(SmemPtr lds, int slot, int *refus
         const bool has_new = uni((int)(a.pos_id >= first_token && a.pos_id < first_token + RUB * NSLOT)) != 0;
         if (has_new) {
 #pragma unroll
-            for (int u = 0; u < RUB; u++) dst[u] = ld_b128(kvb + (size_t)(t0 + min(token_of(rb + u), T - 1)) * tok_stride);
+            for (int u = 0; u < RUB; u++) {
+                const int t = t0 + min(token_of(rb + u), T - 1);
+                dst[u] = staged && t == a.pos_id ? newest_row(kvb) : ld_b128(kvb + (size_t)t * tok_stride);
+            }
         } else {
 #pragma unroll
             for (int u = 0; u < RUB; u++) dst[u] = ld_const_b128(kvb + (size_t)(t0 + min(token_of(rb + u), T - 1)) * tok_stride);
@@ -2759,6 +2877,7 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
         sm->k.argmax = ws + w.argmax;
         sm->k.pads = ws + w.pads;
         sm->k.partial = reinterpret_cast<uint64_t *>(ws + w.partial);
+        sm->k.stamped = reinterpret_cast<uint64_t *>(ws + w.stamped);
         sm->k.epoch = (uint32_t)ld_i32(ws + w.status + kEpochSlot);
         sm->k.trace_base =
             (a.flags & MK_FLAG_TIMINGS) && a.timings ? a.timings + (size_t)blockIdx.x * a.num_slots * MK_TIMING_SLOTS : nullptr;

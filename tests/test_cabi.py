@@ -48,8 +48,9 @@ def test_workspace_size_and_static_queries():
     small = lib.mk_llama_workspace_bytes(16, 2048, 8192, 2048)
     big = lib.mk_llama_workspace_bytes(32, 4096, 14336, 2048)
     # 1B: status padded to a 128-byte line + 4 copies x 16 shards x 16 layers x 4 counters + 1024 x 2 LM-head
-    # maxima + 4 groups x 2048 partial sums as (value, tag) pairs + 16 layers x 2 rows x 48 padded counters
-    assert small == 4 * (32 + 4 * 16 * 16 * 4 + 2 * 1024 + 2 * 4 * 2048 + 16 * 2 * 48 * 32)
+    # maxima + 4 groups x 2048 partial sums as (value, tag) pairs + 16 layers x 2 rows x 48 padded counters + 2048 stamped
+    # pairs (query, K row, V row)
+    assert small == 4 * (32 + 4 * 16 * 16 * 4 + 2 * 1024 + 2 * 4 * 2048 + 16 * 2 * 48 * 32 + 2 * 2048)
     assert big > small and big < (5 << 18)
     assert lib.mk_llama_workspace_bytes(0, 2048, 8192, 2048) == 0
     assert lib.mk_llama_query(3) == 6                      # ABI version
