@@ -156,6 +156,18 @@ constexpr int rows_in_flight(int wanted) { return KC <= 4 ? wanted : (wanted < M
 #ifndef MK_STAGE_QUERY
 #define MK_STAGE_QUERY 1            // attention takes the query and the step's K / V row from their stamped copies
 #endif
+#ifndef MK_HOLD_NOSLEEP
+#define MK_HOLD_NOSLEEP 0
+#endif
+#ifndef MK_HOLD_LOOKS
+#define MK_HOLD_LOOKS 2
+#endif
+#ifndef MK_HOLD_SHARE
+#define MK_HOLD_SHARE 30            // thirty-seconds of the arrivals
+#endif
+#ifndef MK_WIDE_CONTROLLER_CALL
+#define MK_WIDE_CONTROLLER_CALL 1
+#endif
 #ifndef MK_POLL_SLEEP
 #define MK_POLL_SLEEP 10            // units of 64 clocks between two looks at a dependency
 #endif
@@ -225,6 +237,7 @@ struct Consts {
     int pad_cols;                   // padded per-head counters per (layer, row)
     int down_jobs, o_jobs;          // arrivals that complete barrier rows 5 and 3
     int shard_stride, replica_stride;  // ints from one shard / one replica of a sharded counter to the next
+    int hold_looks;                 // looks at a nearly complete dependency before the consumers' bulk requests are released
 };
 // A matvec instruction (opcodes 1, 4, 5, 6) decoded once per launch: where its weight rows live.
 // ntasks < 0: the instruction is malformed.
@@ -670,11 +683,23 @@ __device__ __forceinline__ bool poll_wait(const Ctx &c, PollTicket t, bool sum_m
     const int *status = ws_status(c);
     int v = t.value, st = t.status;
     bool first = true;
+    int held = 0;
+    const int hold_looks = sum_mode ? uni(c.sm->k.hold_looks) : 0;
     while (true) {
-        const bool ok = sum_mode ? (lane_sum_i32(v) >= target) : (bool)__all(t.ptr == nullptr || v + t.base >= target);
+        const int arrived = sum_mode ? lane_sum_i32(v) : 0;
+        const bool ok = sum_mode ? (arrived >= target) : (bool)__all(t.ptr == nullptr || v + t.base >= target);
         if (ok) break;
-        if (first) not_yet();
-        first = false;
+        // Nearly everybody has arrived: the rest is a microsecond away.  The bulk requests that `not_yet`
+        // releases would hold up the next looks and the fetch of the vector behind them (a CU serves its
+        // requests in order), so they wait for up to two more looks - where the step is a chain of
+        // hand-overs (the slowest worker of a phase, which arrives last, sees its dependency 1.5 µs
+        // earlier); where the phases are bounded by memory, holding requests back only loses bandwidth.
+        const bool hold = first && held < hold_looks && arrived * 32 >= target * MK_HOLD_SHARE;
+        if (hold) held++;
+        if (first && !hold) {
+            not_yet();
+            first = false;
+        }
         if (__any(st != 0)) return false;
         if (wall_clock64() - t0 > limit) {
             if (c.lane == 0) record_status(c, MK_STATUS_BARRIER_TIMEOUT);
@@ -682,7 +707,7 @@ __device__ __forceinline__ bool poll_wait(const Ctx &c, PollTicket t, bool sum_m
         }
         // a quarter microsecond between looks: more looks (or two in flight) only add traffic on
         // the counters' memory channels and make the step slower
-        __builtin_amdgcn_s_sleep(MK_POLL_SLEEP);
+        if (!(hold && MK_HOLD_NOSLEEP)) __builtin_amdgcn_s_sleep(MK_POLL_SLEEP);
         v = t.ptr ? ld_i32(t.ptr) : 0;
         st = c.lane == 63 ? ld_i32(status) : 0;
     }
@@ -2610,6 +2635,31 @@ __device__ __forceinline__ bool controller_step(SmemPtr sm, int slot, int opcode
     }
 }
 
+// The same with a function of its own per instruction kind: where the activation vector is 4096 wide,
+// the controller's side of an instruction needs most of the registers, and inlined in the instruction
+// loop (or all kinds in one function) it pushes values into scratch memory.
+template <bool TR, int OP, int KC, bool WIDE>
+static __device__ __noinline__ bool controller_matvec_call(SmemPtr sm, int slot, int *refusal) {
+    return matvec_impl<TR, OP, KC, 0, kControllerRole, 0, false, 0, WIDE>(sm, slot, refusal);
+}
+template <bool TR, int D>
+static __device__ __noinline__ bool controller_attention_call(SmemPtr sm, int slot, int *refusal) {
+    return attention_impl<TR, D, kControllerRole>(sm, slot, refusal);
+}
+template <bool TR, int KC_HID, int KC_RED, int D>
+__device__ __forceinline__ bool controller_step_call(SmemPtr sm, int slot, int opcode, int *refusal) {
+    switch (opcode) {
+    case 1: return controller_matvec_call<TR, 1, KC_HID, true>(sm, slot, refusal);
+    case 2: return controller_attention_call<TR, D>(sm, slot, refusal);
+    case 3: return reduction_impl<TR, D, kControllerRole>(sm, slot, refusal);
+    case 4: return controller_matvec_call<TR, 4, KC_RED, true>(sm, slot, refusal);
+    case 5: return controller_matvec_call<TR, 5, KC_HID, true>(sm, slot, refusal);
+    case 6: return controller_matvec_call<TR, 6, KC_RED, true>(sm, slot, refusal);
+    case 7: return op_lm_head<TR, KC_HID>(sm, slot, refusal);
+    default: return bail(make_ctx<TR>(sm, slot, opcode), MK_STATUS_BAD_OPCODE, refusal);
+    }
+}
+
 // ---------------------------------------------------------------------------------------------
 // the persistent kernel
 // ---------------------------------------------------------------------------------------------
@@ -2888,6 +2938,7 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
         sm->k.o_jobs = (a.hidden_size / a.matvec_reduction_size) * (a.hidden_size / 16);
         sm->k.shard_stride = a.num_layers * kHotRows;
         sm->k.replica_stride = kShards * a.num_layers * kHotRows;
+        sm->k.hold_looks = a.hidden_size != a.matvec_reduction_size ? 0 : MK_HOLD_LOOKS;
     }
     // A launch covers one decode step, or `num_steps` of them back to back: the token a step
     // produces starts the next one, at the next position.
@@ -2936,7 +2987,10 @@ __global__ __launch_bounds__(kThreads) void mk_llama_kernel(const mk_llama_args 
                 }
                 bool ok = true;
                 if (controller) {
-                    ok = uni((int)controller_step<TR, KC_HID, KC_RED, D>(sm, slot, opcode, &refusal)) != 0;
+                    if constexpr (kWide && MK_WIDE_CONTROLLER_CALL)
+                        ok = uni((int)controller_step_call<TR, KC_HID, KC_RED, D>(sm, slot, opcode, &refusal)) != 0;
+                    else
+                        ok = uni((int)controller_step<TR, KC_HID, KC_RED, D>(sm, slot, opcode, &refusal)) != 0;
                 } else switch (opcode) {
                 case 1: ok = uni((int)op_matvec<TR, 1, KC_HID, kWide ? MK_WIDE_PARK_QKV : 0, 0, kWide>(sm, slot, &refusal)) != 0; break;
                 case 2: ok = uni((int)op_attention<TR, D>(sm, slot, &refusal)) != 0; break;
